@@ -101,6 +101,8 @@ extern "C" int rv_gemm_groups_plain(hipStream_t stream, const void* a, int a_dty
       w_group_stride, c_group_stride, (const TC*)gate, ldg)
   if (a_dtype == RV_F32 && w_dtype == RV_F32 && c_dtype == RV_F32) RV_GG(float, float, float);
   else if (a_dtype == RV_BF16 && w_dtype == RV_BF16 && c_dtype == RV_BF16) RV_GG(bf16_t, bf16_t, bf16_t);
+  else if (a_dtype == RV_BF16 && w_dtype == RV_BF16 && c_dtype == RV_F32 && gate == nullptr)
+    RV_GG(bf16_t, bf16_t, float);  // 32-bit sums handed on unrounded
   else return rv_fail("gemm_groups: unsupported dtypes a=%d w=%d c=%d", a_dtype, w_dtype, c_dtype);
 #undef RV_GG
   RV_LAUNCH_CHECK("gemm_groups_plain");
@@ -117,7 +119,8 @@ extern "C" int rv_gemm_groups_plain(hipStream_t stream, const void* a, int a_dty
 //
 // Epilogues: a gate (C * sigmoid(gate)); or, GLU, the clamped gated activation of an expert applied where the sums
 // are held: W holds N gate rows and then N up rows, the wave multiplies both against the same tokens and writes
-// g * sigmoid(alpha g) * (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit): the expert's inner
+// g * sigmoid(alpha g) * (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit) (glu 1), or the plain
+// silu(gate) * up (glu 2: no limit, alpha 1, the up as it is): the expert's inner
 // activations never exist unactivated in memory.
 // ---------------------------------------------------------------------------
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 gg_bf16x8;
@@ -137,6 +140,7 @@ struct GroupsParams {
   int M, N, K;
   long long lda, ldw, ldc, ldg, a_group_stride, w_group_stride, c_group_stride;
   float limit, alpha;
+  float up_offset;  // what the clamped up is raised by: 1 in the clamped form, 0 in the plain one
   int vec_store;
 };
 
@@ -251,7 +255,7 @@ __global__ void __launch_bounds__(256) gemm_groups_mfma_kernel(const GroupsParam
         if constexpr (GLU) {
           const float g = fminf(v[i], P.limit);
           const float u = fminf(fmaxf(acc_up[mt][t][i], -P.limit), P.limit);
-          v[i] = g * (u + 1.0f) * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * P.alpha * g));
+          v[i] = g * (u + P.up_offset) * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * P.alpha * g));
         }
         if (gr != nullptr && n + i < P.N) {
           const float z = __uint_as_float(((uint32_t)gr[n + i]) << 16);
@@ -399,7 +403,7 @@ __global__ void __launch_bounds__(256) gemm_experts_lds_kernel(const GroupsParam
         if constexpr (GLU) {
           const float g = fminf(v[i], P.limit);
           const float u = fminf(fmaxf(acc[mt][t + 2][i], -P.limit), P.limit);
-          v[i] = g * (u + 1.0f) * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * P.alpha * g));
+          v[i] = g * (u + P.up_offset) * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * P.alpha * g));
         }
       }
       if (P.vec_store && n + 3 < P.N) {
@@ -431,7 +435,8 @@ extern "C" int rv_gemm_groups_mfma(hipStream_t stream, const void* a, const void
            "gemm_groups_mfma: K, the rows' strides and the groups' strides must be multiples of 8 and the operands "
            "16-byte aligned");
   RV_CHECK(lda >= K && ldw >= K && ldc >= N && (gate == nullptr || ldg >= N), "gemm_groups_mfma: rows too short");
-  RV_CHECK(!glu || (gate == nullptr && limit > 0.f), "gemm_groups_mfma: the gated activation takes a limit and no gate");
+  RV_CHECK(!glu || (gate == nullptr && (glu == 2 || limit > 0.f)),
+           "gemm_groups_mfma: the gated activation takes a limit and no gate");
   RV_CHECK(token_tiles == 1 || token_tiles == 4, "gemm_groups_mfma: 1 or 4 tiles of 16 tokens a wave, not %d", token_tiles);
   if (M == 0) return 0;
   GroupsParams P;
@@ -444,7 +449,8 @@ extern "C" int rv_gemm_groups_mfma(hipStream_t stream, const void* a, const void
   P.M = M, P.N = N, P.K = K;
   P.lda = lda, P.ldw = ldw, P.ldc = ldc, P.ldg = ldg;
   P.a_group_stride = a_group_stride, P.w_group_stride = w_group_stride, P.c_group_stride = c_group_stride;
-  P.limit = limit, P.alpha = alpha;
+  P.limit = limit, P.alpha = alpha, P.up_offset = 1.0f;
+  if (glu == 2) P.limit = __builtin_inff(), P.alpha = 1.0f, P.up_offset = 0.0f;  // silu(gate) * up, nothing clamped
   P.vec_store = (ldc % 4 == 0 && c_group_stride % 4 == 0 && ((uintptr_t)c & 7) == 0) ? 1 : 0;
   if (groups == 0 && token_tiles == 4 && gate == nullptr) {  // the experts' products of many rows: tiles through LDS
     dim3 grid(rv_div_up(N, glu ? GL_BW / 2 : GL_BW), rv_div_up(M, GL_BM)), block(256);

@@ -128,3 +128,93 @@ extern "C" int rv_moe_combine(hipStream_t stream, const void* y, const int* slot
   RV_LAUNCH_CHECK("moe_combine");
   return 0;
 }
+
+// ---------------------------------------------------------------------------
+// Routing by the activations: a router's 32-bit logits [tokens, experts] give every token the `top` experts with
+// the largest logits (the largest first; of equal ones the lower index), each with the weight sigmoid(logit) (mode
+// 0).  A wave a token: every lane holds the logits e * 64 + lane, the largest is found by a sum-free exchange
+// (value, then index) and struck out, `top` times.  The result, chosen [tokens, top], is a table for moe_route
+// with the token's row as its id.
+// ---------------------------------------------------------------------------
+#define MOE_TOPK_PER (MOE_MAX_EXPERTS / RV_WAVE)
+
+__global__ void __launch_bounds__(256)
+moe_topk_kernel(const float* __restrict__ logits, int num_tokens, int experts, int top, int* __restrict__ chosen,
+                float* __restrict__ weights) {
+  const int lane = threadIdx.x & (RV_WAVE - 1);
+  const int t = blockIdx.x * (blockDim.x / RV_WAVE) + threadIdx.x / RV_WAVE;
+  if (t >= num_tokens) return;  // the whole wave
+  const float* row = logits + (size_t)t * experts;
+  float v[MOE_TOPK_PER];
+#pragma unroll
+  for (int e = 0; e < MOE_TOPK_PER; ++e) {
+    const int i = e * RV_WAVE + lane;
+    const float x = i < experts ? row[i] : -INFINITY;
+    v[e] = x == x ? x : -INFINITY;  // a NaN is never chosen
+  }
+  for (int k = 0; k < top; ++k) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+#pragma unroll
+    for (int e = 0; e < MOE_TOPK_PER; ++e) {
+      const int i = e * RV_WAVE + lane;
+      if (i < experts && (v[e] > best || (v[e] == best && i < at))) best = v[e], at = i;
+    }
+#pragma unroll
+    for (int off = RV_WAVE / 2; off > 0; off >>= 1) {
+      const float ob = __shfl_xor(best, off, RV_WAVE);
+      const int oa = __shfl_xor(at, off, RV_WAVE);
+      if (ob > best || (ob == best && oa < at)) best = ob, at = oa;
+    }
+    if (at >= experts) at = k;  // nothing left to choose from (every logit NaN or struck out): any expert, weight 0
+    if (lane == 0) {
+      chosen[(size_t)t * top + k] = at;
+      weights[(size_t)t * top + k] = best > -INFINITY ? 1.0f / (1.0f + expf(-best)) : 0.f;
+    }
+#pragma unroll
+    for (int e = 0; e < MOE_TOPK_PER; ++e)
+      if (e * RV_WAVE + lane == at) v[e] = -INFINITY;
+  }
+}
+
+extern "C" int rv_moe_topk(hipStream_t stream, const float* logits, int num_tokens, int experts, int top, int* chosen,
+                           float* weights) {
+  RV_CHECK(logits && chosen && weights && num_tokens >= 0, "moe_topk: bad arguments");
+  RV_CHECK(experts > 0 && experts <= MOE_MAX_EXPERTS && top > 0 && top <= experts,
+           "moe_topk: %d of %d experts (at most %d)", top, experts, MOE_MAX_EXPERTS);
+  if (num_tokens == 0) return 0;
+  moe_topk_kernel<<<dim3(rv_div_up(num_tokens, 4)), dim3(256), 0, stream>>>(logits, num_tokens, experts, top, chosen,
+                                                                            weights);
+  RV_LAUNCH_CHECK("moe_topk");
+  return 0;
+}
+
+// xs[slot_of[p]] = weights[p] * x[p / top], rounded to T: the rows of the experts' first product where a choice's
+// weight multiplies the expert's input.  A block a (token, choice) pair; a pair without a row is skipped; rows of
+// xs that no pair names are left as they are.
+template <typename T>
+__global__ void moe_scale_rows_kernel(const T* __restrict__ x, const int* __restrict__ slot_of,
+                                      const float* __restrict__ weights, int top, T* __restrict__ xs, int width) {
+  const int p = blockIdx.x;
+  const int row = slot_of[p];
+  if (row < 0) return;
+  const float w = weights[p];
+  const T* src = x + (size_t)(p / top) * width;
+  T* dst = xs + (size_t)row * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = rv_from_float<T>(w * rv_to_float(src[i]));
+}
+
+extern "C" int rv_moe_scale_rows(hipStream_t stream, const void* x, const int* slot_of, const float* weights, int top,
+                                 void* xs, int dtype, int num_tokens, int width) {
+  RV_CHECK(x && slot_of && weights && xs && num_tokens >= 0 && top > 0 && width > 0, "moe_scale_rows: bad arguments");
+  if (num_tokens == 0) return 0;
+  dim3 grid(num_tokens * top), block(256);
+  if (dtype == RV_F32)
+    moe_scale_rows_kernel<float><<<grid, block, 0, stream>>>((const float*)x, slot_of, weights, top, (float*)xs, width);
+  else if (dtype == RV_BF16)
+    moe_scale_rows_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)x, slot_of, weights, top, (bf16_t*)xs, width);
+  else
+    return rv_fail("moe_scale_rows: unsupported dtype %d", dtype);
+  RV_LAUNCH_CHECK("moe_scale_rows");
+  return 0;
+}

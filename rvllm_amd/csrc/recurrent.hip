@@ -71,7 +71,8 @@ causal_conv_kernel(const T* __restrict__ in, long long ld_in, const float* __res
                    int state_ld, const int* __restrict__ positions, const int* __restrict__ token_req,
                    const int* __restrict__ q_start, const int* __restrict__ chunk_start,
                    const int* __restrict__ state_slot, TO* __restrict__ out, long long ld_out, int channels, int group,
-                   int groups, int num_tokens, float unit_eps, int scaled_groups, float group_scale, int move_state) {
+                   int groups, int num_tokens, float unit_eps, int scaled_groups, float group_scale, int move_state,
+                   int act) {
   const int lane = threadIdx.x & (RV_WAVE - 1);
   const long long unit = (long long)blockIdx.x * (blockDim.x / RV_WAVE) + threadIdx.x / RV_WAVE;
   if (unit >= (long long)num_tokens * groups) return;  // the whole wave
@@ -93,7 +94,7 @@ causal_conv_kernel(const T* __restrict__ in, long long ld_in, const float* __res
                                : st[(long long)(taps - 1 + r) * state_ld + c];
         acc = fmaf(w[(long long)c * taps + j], x, acc);
       }
-      const float y = rv_round_to<T>(rec_silu(acc));
+      const float y = rv_round_to<T>(act == 0 ? rec_silu(acc) : acc);
       if (unit_eps < 0.f) {
         out[(long long)t * ld_out + c] = rv_from_float<TO>(y);
         if (move_state) {  // rel is 0: rows 1 .. taps - 2 move up, the token's input goes last
@@ -117,7 +118,7 @@ causal_conv_kernel(const T* __restrict__ in, long long ld_in, const float* __res
                                : st[(long long)(taps - 1 + r) * state_ld + c];
         acc = fmaf(w[(long long)c * taps + j], x, acc);
       }
-      out[(long long)t * ld_out + c] = rv_from_float<TO>(rv_round_to<T>(rec_silu(acc)) * mult);
+      out[(long long)t * ld_out + c] = rv_from_float<TO>(rv_round_to<T>(act == 0 ? rec_silu(acc) : acc) * mult);
       if (move_state) {
         for (int s_ = 0; s_ + 2 < taps; ++s_) st[(long long)s_ * state_ld + c] = st[(long long)(s_ + 1) * state_ld + c];
         if (taps > 1) st[(long long)(taps - 2) * state_ld + c] = rv_to_float(in[(long long)first_tok * ld_in + c]);
@@ -128,17 +129,18 @@ causal_conv_kernel(const T* __restrict__ in, long long ld_in, const float* __res
 
 // in: [tokens, ld_in] of type `dtype`, the channels from the given address on.  w: float [channels, taps]; bias:
 // float [channels] or null.  state: float, row s of a slot's block at state_off + s * state_ld.  out: float
-// (out_f32) or `dtype`.  unit_eps < 0: no unit length.
+// (out_f32) or `dtype`.  unit_eps < 0: no unit length.  act 0: silu, 1: none.
 extern "C" int rv_causal_conv(hipStream_t stream, const void* in, int dtype, long long ld_in, const float* w,
                               const float* bias, int taps, float* state, long long slot_stride,
                               long long state_off, int state_ld, const int* positions, const int* token_req,
                               const int* q_start, const int* chunk_start, const int* state_slot, void* out,
                               int out_f32, long long ld_out, int channels, int group, int num_tokens, float unit_eps,
-                              int scaled_groups, float group_scale, int move_state) {
+                              int scaled_groups, float group_scale, int move_state, int act) {
   RV_CHECK(in && w && state && positions && token_req && q_start && chunk_start && state_slot && out,
            "causal_conv: null argument");
   RV_CHECK(taps >= 1 && taps <= REC_MAX_TAPS && channels > 0 && group > 0 && num_tokens >= 0 && state_ld >= channels,
            "causal_conv: bad sizes taps=%d channels=%d group=%d", taps, channels, group);
+  RV_CHECK(act == 0 || act == 1, "causal_conv: activation %d (0: silu, 1: none)", act);
   if (num_tokens == 0) return 0;
   const int groups = rv_div_up(channels, group);
   const long long units = (long long)num_tokens * groups;
@@ -148,7 +150,7 @@ extern "C" int rv_causal_conv(hipStream_t stream, const void* in, int dtype, lon
                                                         state_off, state_ld, positions, token_req, q_start,          \
                                                         chunk_start, state_slot, (TO*)out, ld_out, channels, group,  \
                                                         groups, num_tokens, unit_eps, scaled_groups, group_scale,     \
-                                                        move_state)
+                                                        move_state, act)
   if (dtype == RV_F32) RV_CC(float, float);
   else if (dtype == RV_BF16 && out_f32) RV_CC(bf16_t, float);
   else if (dtype == RV_BF16) RV_CC(bf16_t, bf16_t);
@@ -610,13 +612,15 @@ extern "C" int rv_selective_scan(hipStream_t stream, const void* x, long long ld
 }
 
 // ---------------------------------------------------------------------------
-// out[t][h][:] = o[t][h][:] / sqrt(mean(o[t][h][:]^2) + eps) * w[:] * silu(gate[t][h][:]); a wave a (token, head).
-// o: float [tokens, heads dv]; gate: T, rows ld_gate apart; w: float [dv], shared by the heads; out: T.
+// out[t][h][:] = o[t][h][:] / sqrt(mean(o[t][h][:]^2) + eps) * w[:] * act(gate[t][h][:]); a wave a (token, head).
+// o: float [tokens, heads dv]; gate: T, rows ld_gate apart; w: float [dv], shared by the heads, or (w_per_head)
+// [heads dv], every head its own; act 0: sigmoid, 1: silu; out: T.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ void __launch_bounds__(256)
 head_norm_gate_kernel(const float* __restrict__ o, const T* __restrict__ gate, long long ld_gate,
-                      const float* __restrict__ w, T* __restrict__ out, int heads, int dv, float eps, long long units) {
+                      const float* __restrict__ w, T* __restrict__ out, int heads, int dv, float eps, long long units,
+                      int w_per_head, int act) {
   const int lane = threadIdx.x & (RV_WAVE - 1);
   const long long unit = (long long)blockIdx.x * (blockDim.x / RV_WAVE) + threadIdx.x / RV_WAVE;
   if (unit >= units) return;
@@ -629,22 +633,25 @@ head_norm_gate_kernel(const float* __restrict__ o, const T* __restrict__ gate, l
   const float inv = 1.0f / sqrtf(ss / (float)dv + eps);
   for (int d = lane; d < dv; d += RV_WAVE) {
     const float gv = rv_to_float(gate[t * ld_gate + (long long)h * dv + d]);
-    out[unit * dv + d] = rv_from_float<T>(row[d] * inv * w[d] * rec_silu(gv));
+    const float wv = w[w_per_head ? (long long)h * dv + d : d];
+    out[unit * dv + d] = rv_from_float<T>(row[d] * inv * wv * (act == 0 ? rec_sigmoid(gv) : rec_silu(gv)));
   }
 }
 
 extern "C" int rv_head_norm_gate(hipStream_t stream, const float* o, const void* gate, long long ld_gate,
-                                 const float* w, void* out, int dtype, int num_tokens, int heads, int dv, float eps) {
-  RV_CHECK(o && gate && w && out && heads > 0 && dv > 0 && num_tokens >= 0, "head_norm_gate: bad arguments");
+                                 const float* w, void* out, int dtype, int num_tokens, int heads, int dv, float eps,
+                                 int w_per_head, int act) {
+  RV_CHECK(o && gate && w && out && heads > 0 && dv > 0 && num_tokens >= 0 && (act == 0 || act == 1),
+           "head_norm_gate: bad arguments");
   if (num_tokens == 0) return 0;
   const long long units = (long long)num_tokens * heads;
   dim3 grid(rv_div_up(units, 4)), block(256);
   if (dtype == RV_F32)
     head_norm_gate_kernel<float><<<grid, block, 0, stream>>>(o, (const float*)gate, ld_gate, w, (float*)out, heads, dv,
-                                                             eps, units);
+                                                             eps, units, w_per_head, act);
   else if (dtype == RV_BF16)
     head_norm_gate_kernel<bf16_t><<<grid, block, 0, stream>>>(o, (const bf16_t*)gate, ld_gate, w, (bf16_t*)out, heads,
-                                                              dv, eps, units);
+                                                              dv, eps, units, w_per_head, act);
   else
     return rv_fail("head_norm_gate: unsupported dtype %d", dtype);
   RV_LAUNCH_CHECK("head_norm_gate");

@@ -4,7 +4,9 @@
 //
 //   rotation  (u, v) = (x[i], x[i + rot/2]) -> (u cos a - v sin a, v cos a + u sin a), a = position * f_i, i < rot/2;
 //             dimensions from `rot` on pass unchanged.  cos and sin come from the step's 32-bit table.
-//   norm      x / sqrt(mean(x^2) + eps) * (offset + w[d]) over the head's `hd` dimensions; w null: no weight;
+//   norm      x / sqrt(mean(x^2) + eps) * (offset + w[d]) over the head's first `norm_dim` dimensions (all of them,
+//             unless the head is stored wider than it is, with zeros behind: then the mean is over the head's own
+//             size and the zeros stay zeros); w null: no weight;
 //             norm_mode 0: none, 1: before the rotation, 2: after it
 //   write     queries to q_out [tokens, nq * hd]; keys (rotated, normed) and values into the paged cache of
 //             kv_layout.h at the token's position; a negative page skips the write.  v_col < 0: the value is the
@@ -27,7 +29,7 @@ rotate_norm_write_kernel(const T* __restrict__ in, long long ld, int q_col, int 
                          const float* __restrict__ sin_t, int rot, const int* __restrict__ positions,
                          const int* __restrict__ token_req, const int* __restrict__ table, int table_width,
                          T* __restrict__ k_pages, T* __restrict__ v_pages, int page_size, int num_pages, int num_tokens,
-                         int nq, int nkv, int hd, int write_kv) {
+                         int nq, int nkv, int hd, int write_kv, int norm_dim) {
   const int lane = threadIdx.x & (RV_WAVE - 1);
   const long long unit = (long long)blockIdx.x * (blockDim.x / RV_WAVE) + threadIdx.x / RV_WAVE;
   const int per_token = nq + nkv;
@@ -51,13 +53,13 @@ rotate_norm_write_kernel(const T* __restrict__ in, long long ld, int q_col, int 
     ss_raw = fmaf(raw[e], raw[e], ss_raw);
   }
   float inv_before = 1.0f;
-  if (norm_mode == 1) inv_before = 1.0f / sqrtf(rv_wave_sum(ss_raw) / (float)hd + eps);
+  if (norm_mode == 1) inv_before = 1.0f / sqrtf(rv_wave_sum(ss_raw) / (float)norm_dim + eps);
   float ss = 0.f;
 #pragma unroll
   for (int e = 0; e < RNW_E; ++e) {
     const int d = e * RV_WAVE + lane;
     float x = raw[e];
-    if (norm_mode == 1 && d < hd) x *= inv_before * (w ? offset + rv_load_w(w, w_f32, d) : 1.0f);
+    if (norm_mode == 1 && d < norm_dim) x *= inv_before * (w ? offset + rv_load_w(w, w_f32, d) : 1.0f);
     if (d < rot) {
       const int partner = d < half ? d + half : d - half;
       float y = b ? rv_round_to<T>(rv_to_float(src[partner]) + b[partner]) : rv_to_float(src[partner]);
@@ -70,11 +72,11 @@ rotate_norm_write_kernel(const T* __restrict__ in, long long ld, int q_col, int 
     ss = fmaf(x, x, ss);
   }
   if (norm_mode == 2) {
-    const float inv = 1.0f / sqrtf(rv_wave_sum(ss) / (float)hd + eps);
+    const float inv = 1.0f / sqrtf(rv_wave_sum(ss) / (float)norm_dim + eps);
 #pragma unroll
     for (int e = 0; e < RNW_E; ++e) {
       const int d = e * RV_WAVE + lane;
-      if (d < hd) val[e] *= inv * (w ? offset + rv_load_w(w, w_f32, d) : 1.0f);
+      if (d < norm_dim) val[e] *= inv * (w ? offset + rv_load_w(w, w_f32, d) : 1.0f);
     }
   }
   if (is_q) {
@@ -108,13 +110,15 @@ extern "C" int rv_rotate_norm_write(hipStream_t stream, const void* in, long lon
                                     int norm_mode, const float* cos_t, const float* sin_t, int rot,
                                     const int* positions, const int* token_req, const int* table, int table_width,
                                     void* k_pages, void* v_pages, int page_size, int num_pages, int dtype,
-                                    int num_tokens, int nq, int nkv, int hd, int write_kv) {
+                                    int num_tokens, int nq, int nkv, int hd, int write_kv, int norm_dim) {
   RV_CHECK(in && q_out && positions && token_req, "rotate_norm_write: null argument");
   RV_CHECK(nq > 0 && nkv > 0 && hd > 0 && hd <= RNW_MAX_HD, "rotate_norm_write: head size %d must be at most %d", hd,
            RNW_MAX_HD);
   RV_CHECK(rot >= 0 && rot <= hd && rot % 2 == 0 && (rot == 0 || (cos_t && sin_t)),
            "rotate_norm_write: %d rotated dimensions of %d need an even count and the step's table", rot, hd);
   RV_CHECK(norm_mode >= 0 && norm_mode <= 2, "rotate_norm_write: norm_mode %d", norm_mode);
+  RV_CHECK(norm_dim >= rot && norm_dim >= 1 && norm_dim <= hd,
+           "rotate_norm_write: the norm runs over %d of a head's %d dimensions, %d of them rotated", norm_dim, hd, rot);
   RV_CHECK(!write_kv || (table && k_pages && v_pages && page_size > 0 && page_size % RV_V_GROUP == 0),
            "rotate_norm_write: no cache to write to");
   if (num_tokens == 0) return 0;
@@ -124,7 +128,7 @@ extern "C" int rv_rotate_norm_write(hipStream_t stream, const void* in, long lon
   rotate_norm_write_kernel<T><<<grid, block, 0, stream>>>((const T*)in, ld, q_col, k_col, v_col, bias, (T*)q_out, q_w, k_w, \
                                                           w_f32, eps, offset, norm_mode, cos_t, sin_t, rot, positions, \
                                                           token_req, table, table_width, (T*)k_pages, (T*)v_pages,     \
-                                                          page_size, num_pages, num_tokens, nq, nkv, hd, write_kv)
+                                                          page_size, num_pages, num_tokens, nq, nkv, hd, write_kv, norm_dim)
   if (dtype == RV_F32) RV_RNW(float);
   else if (dtype == RV_BF16) RV_RNW(bf16_t);
   else return rv_fail("rotate_norm_write: unsupported dtype %d", dtype);

@@ -386,12 +386,13 @@ def moe_route(token_ids: torch.Tensor, num_tokens: int, table: torch.Tensor, exp
 
 def gemm_experts(a: torch.Tensor, w: torch.Tensor, tile_group: torch.Tensor, row_index: Optional[torch.Tensor] = None,
                  out: Optional[torch.Tensor] = None, tile: int = MOE_TILE_ROWS, mfma: bool = False,
-                 glu: Optional[tuple[float, float]] = None) -> torch.Tensor:
+                 glu=None) -> torch.Tensor:
     """``out[r] = a[row_index[r]] @ w[tile_group[r // tile]]^T`` for the sorted rows of ``moe_route``; ``w`` is
     ``[experts, N, K]``.  Without ``row_index`` the rows of ``a`` are the sorted rows themselves.  Rows of tiles
     without an expert are left as they are.  ``tile`` and ``mfma`` are the step's plan (``moe_plan``).  ``glu`` =
     (limit, alpha), on the matrix cores only: ``w`` holds each expert's gate rows and then its up rows, and the
-    result is the clamped gated activation of the two products, ``[rows, N / 2]``."""
+    result is the clamped gated activation of the two products, ``[rows, N / 2]``; ``glu`` = ``"silu"``: the plain
+    silu(gate) * up instead."""
     _gpu(a, w, tile_group, row_index, out)
     _i32(tile_group)
     _need(a.dim() == 2 and w.dim() == 3 and a.dtype == w.dtype and a.dtype in _DT and a.shape[1] == w.shape[2],
@@ -413,11 +414,12 @@ def gemm_experts(a: torch.Tensor, w: torch.Tensor, tile_group: torch.Tensor, row
     if mfma:
         _need(a.dtype == torch.bfloat16 and _mfma_groups_take(a.data_ptr(), a.stride(0), w, k),
               "gemm_experts: the matrix-core kernel takes bf16 and sizes that are multiples of 8")
-        limit, alpha = glu if glu is not None else (0.0, 0.0)
+        kind = 0 if glu is None else (2 if glu == "silu" else 1)
+        limit, alpha = glu if kind == 1 else (0.0, 0.0)
         _check(library().rv_gemm_groups_mfma(
             _stream(), _ptr(a), _ptr(w), _ptr(out), _ptr(row_index), _ptr(tile_group), _c_int(0), _c_int(m), _c_int(n),
             _c_int(k), _c_ll(a.stride(0)), _c_ll(k), _c_ll(n), _c_ll(0), _c_ll(w.shape[1] * k), _c_ll(0), None, _c_ll(0),
-            _c_int(int(glu is not None)), _c_float(limit), _c_float(alpha), _c_int(tile // 16)))
+            _c_int(kind), _c_float(limit), _c_float(alpha), _c_int(tile // 16)))
         return out
     _check(library().rv_gemm_groups_plain(
         _stream(), _ptr(a), _dt(a), _ptr(w), _dt(w), _ptr(out), _dt(out), _ptr(row_index), _ptr(tile_group), _c_int(0),
@@ -1472,12 +1474,14 @@ def rotate_norm_write(proj: torch.Tensor, q_col: int, k_col: int, v_col: Optiona
                       positions: torch.Tensor, token_req: torch.Tensor, block_table: Optional[torch.Tensor],
                       k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], num_q_heads: int,
                       num_kv_heads: int, head_dim: int, write_kv: bool = True,
-                      bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      bias: Optional[torch.Tensor] = None, norm_dim: Optional[int] = None) -> torch.Tensor:
     """Queries and keys from the rows of ``proj`` (queries from column ``q_col``, keys from ``k_col``, values from
     ``v_col`` or, with None, the keys as they stand there): rotation of the first ``rotary_dim`` dimensions of a
     head, dimension i paired with i + rotary_dim / 2; per-head RMS norm before or after it (``norm_mode``), with
     the weights or without; queries to ``q_out``, keys and values into the cache.  ``bias``: one 32-bit number
-    for every column of ``proj``, added to queries, keys and values as they are read."""
+    for every column of ``proj``, added to queries, keys and values as they are read.  ``norm_dim``: the head's own
+    size where it is stored wider than it is, with zeros behind (the norm's mean runs over that many)."""
+    norm_dim = head_dim if norm_dim is None else int(norm_dim)
     cos, sin = rope if rope is not None else (None, None)
     _gpu(q_out, q_weight, k_weight, cos, sin, positions, token_req, block_table, k_pages, v_pages, bias)
     _need(bias is None or (bias.dtype == torch.float32 and bias.shape == (proj.shape[1],)),
@@ -1493,8 +1497,8 @@ def rotate_norm_write(proj: torch.Tensor, q_col: int, k_col: int, v_col: Optiona
     _need(positions.numel() >= n and token_req.numel() >= n, "rotate_norm_write: positions/token_req too short")
     w_f32 = 0
     if q_weight is not None or k_weight is not None:
-        _need(q_weight is not None and k_weight is not None and q_weight.shape == (head_dim,)
-              and k_weight.shape == (head_dim,) and q_weight.dtype == k_weight.dtype and q_weight.dtype in _DT,
+        _need(q_weight is not None and k_weight is not None and q_weight.shape == (norm_dim,)
+              and k_weight.shape == (norm_dim,) and q_weight.dtype == k_weight.dtype and q_weight.dtype in _DT,
               "rotate_norm_write: bad norm weights")
         w_f32 = int(q_weight.dtype == torch.float32)
     rot = rotary_dim if rope is not None else 0
@@ -1515,7 +1519,7 @@ def rotate_norm_write(proj: torch.Tensor, q_col: int, k_col: int, v_col: Optiona
         _ptr(bias), _ptr(q_out), _ptr(q_weight), _ptr(k_weight), _c_int(w_f32), _c_float(eps), _c_float(offset), _c_int(norm_mode),
         _ptr(cos), _ptr(sin), _c_int(rot), _ptr(positions), _ptr(token_req), _ptr(block_table), _c_int(width),
         _ptr(k_pages), _ptr(v_pages), _c_int(page_size), _c_int(num_pages), _dt(proj), _c_int(n), _c_int(num_q_heads),
-        _c_int(num_kv_heads), _c_int(head_dim), _c_int(int(write_kv))))
+        _c_int(num_kv_heads), _c_int(head_dim), _c_int(int(write_kv)), _c_int(norm_dim)))
     return q_out
 
 
@@ -1542,11 +1546,14 @@ def _state_args(slots: torch.Tensor, what: str) -> int:
     return slots.stride(0)
 
 
+CONV_ACTS = {"silu": 0, "none": 1}
+
+
 def causal_conv(x: torch.Tensor, col0: int, channels: int, weight: torch.Tensor, bias: Optional[torch.Tensor],
                 slots: torch.Tensor, state_off: int, step, out: torch.Tensor, out_col0: int = 0, group: int = 64,
                 unit_eps: Optional[float] = None, scaled_groups: int = 0, group_scale: float = 1.0,
-                state_ld: Optional[int] = None, move_state: bool = False) -> torch.Tensor:
-    """Short causal convolution over time and silu for the channels ``col0 .. col0 + channels`` of the rows of
+                state_ld: Optional[int] = None, move_state: bool = False, act: str = "silu") -> torch.Tensor:
+    """Short causal convolution over time and ``act`` (``silu``, or ``none``) for the channels ``col0 .. col0 + channels`` of the rows of
     ``x``: ``weight`` is float32 ``[channels, taps]`` (the last tap is the token's own), ``bias`` float32 or None.
     The inputs before a request's first token of the step come from its state slot (``taps - 1`` rows of
     ``channels`` floats from ``state_off`` on), which this call only reads (``conv_state_update`` moves it on).
@@ -1557,6 +1564,7 @@ def causal_conv(x: torch.Tensor, col0: int, channels: int, weight: torch.Tensor,
     moves the state on for these channels; only for a step in which every request brings exactly one token (see
     ``conv_moves_state``), where it replaces ``conv_state_update``."""
     _gpu(weight, bias)
+    _need(act in CONV_ACTS, f"causal_conv: unknown activation {act!r}")
     _need(not move_state or step.max_portion == 1, "causal_conv: the state moves with the kernel in steps of single tokens only")
     state_ld = channels if state_ld is None else int(state_ld)
     _need(x.is_cuda and x.dim() == 2 and x.stride(1) == 1 and out.is_cuda and out.dim() == 2 and out.stride(1) == 1,
@@ -1581,7 +1589,7 @@ def causal_conv(x: torch.Tensor, col0: int, channels: int, weight: torch.Tensor,
         out.data_ptr() + out_col0 * out.element_size(), _c_int(out.dtype == torch.float32 and x.dtype != torch.float32),
         _c_ll(out.stride(0)), _c_int(channels), _c_int(group), _c_int(n),
         _c_float(-1.0 if unit_eps is None else unit_eps), _c_int(scaled_groups), _c_float(group_scale),
-        _c_int(int(move_state))))
+        _c_int(int(move_state)), _c_int(CONV_ACTS[act])))
     return out
 
 
@@ -1635,18 +1643,22 @@ def delta_rule(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, ab: torch.
 
 
 def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, gate_col0: int, weight: torch.Tensor, eps: float, heads: int,
-                   dv: int, out_dtype: torch.dtype) -> torch.Tensor:
-    """out[t, h] = o[t, h] / rms(o[t, h]) * weight * silu(gate[t, gate_col0 + h dv ...]) for every head."""
+                   dv: int, out_dtype: torch.dtype, act: str = "silu") -> torch.Tensor:
+    """out[t, h] = o[t, h] / rms(o[t, h]) * weight * act(gate[t, gate_col0 + h dv ...]) for every head; ``weight`` is
+    ``[dv]``, shared by the heads, or ``[heads * dv]``, every head its own; ``act`` is ``silu`` or ``sigmoid``."""
     _gpu(o, weight)
     n = o.shape[0]
     _need(o.dtype == torch.float32 and o.shape == (n, heads * dv), "head_norm_gate: float32 [tokens, heads * dv]")
-    _need(weight.shape == (dv,) and weight.dtype == torch.float32, "head_norm_gate: a float32 weight of the head's size")
+    _need(weight.shape in ((dv,), (heads * dv,)) and weight.dtype == torch.float32,
+          "head_norm_gate: a float32 weight of the head's size, or of all heads' size")
+    _need(act in GATE_ACTS, f"head_norm_gate: unknown activation {act!r}")
+    per_head = int(weight.shape[0] != dv)
     _need(gate.is_cuda and gate.dim() == 2 and gate.stride(1) == 1 and gate.dtype == out_dtype and gate.shape[0] == n
           and 0 <= gate_col0 and gate_col0 + heads * dv <= gate.shape[1], "head_norm_gate: the gate lies outside its rows")
     out = torch.empty((n, heads * dv), dtype=out_dtype, device=o.device)
     _check(library().rv_head_norm_gate(_stream(), _ptr(o), gate.data_ptr() + gate_col0 * gate.element_size(),
                                        _c_ll(gate.stride(0)), _ptr(weight), _ptr(out), _dt(out), _c_int(n), _c_int(heads),
-                                       _c_int(dv), _c_float(eps)))
+                                       _c_int(dv), _c_float(eps), _c_int(per_head), _c_int(GATE_ACTS[act])))
     return out
 
 
@@ -1679,3 +1691,195 @@ def selective_scan(x: torch.Tensor, z: torch.Tensor, z_col0: int, dt: torch.Tens
         _ptr(D), _ptr(slots), _c_ll(stride), _c_ll(state_off), _ptr(step.q_start), _ptr(step.state_slot), _ptr(out),
         _dt(x), _c_int(step.num_requests), _c_int(channels), _c_int(n_state), _c_int(step.max_portion)))
     return out
+
+
+# ---- layer norm, and a residual stream kept in several copies -----------------------------------------------------
+def layernorm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float, out_dtype: torch.dtype,
+              rows: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """(x - mean) / sqrt(variance + eps) * weight + bias over the last dimension, in 32-bit; ``x`` is 32-bit or of
+    ``out_dtype``.  With ``rows`` (int32) the rows ``x[rows]``."""
+    _gpu(x, weight, bias, rows, out)
+    _need(x.dim() == 2 and x.is_contiguous() and x.dtype in _DT, "layernorm: a contiguous matrix expected")
+    width = x.shape[1]
+    _need(weight.shape == (width,) and bias.shape == (width,) and weight.dtype == bias.dtype and weight.dtype in _DT,
+          "layernorm: a weight and a bias of the row's width and of one type")
+    n = x.shape[0]
+    if rows is not None:
+        _i32(rows)
+        n = rows.numel()
+    if out is None:
+        out = torch.empty((n, width), dtype=out_dtype, device=x.device)
+    _need(out.shape == (n, width) and out.dtype == out_dtype and out.is_contiguous(), "layernorm: bad out")
+    _check(library().rv_layernorm(_stream(), _ptr(x), _dt(x), _ptr(rows), _ptr(weight), _ptr(bias),
+                                  _c_int(weight.dtype == torch.float32), _ptr(out), _dt(out), _c_int(n), _c_int(width),
+                                  _c_float(eps)))
+    return out
+
+
+def streams_update(streams: torch.Tensor, out_dtype: torch.dtype, *, seed: Optional[torch.Tensor] = None, branch=None,
+                   layer_scale: Optional[torch.Tensor] = None, mix: Optional[torch.Tensor] = None,
+                   out_w: Optional[torch.Tensor] = None, mult: float = 1.0, in_w: Optional[torch.Tensor] = None,
+                   norm_w: Optional[torch.Tensor] = None, norm_b: Optional[torch.Tensor] = None, eps: float = 0.0,
+                   total: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """One sublayer's turn on the ``streams [S, tokens, width]`` (32-bit, in place) of a model that keeps S copies of
+    its residual stream.  With ``seed`` all copies are first set to it.  With ``branch`` (the sublayer's result: a
+    tensor of ``out_dtype``, ``SlicedSums`` or a ``BranchSum``), all streams at once from the old ones:
+    x_t <- sum_s mix[s, t] x_s + mult * out_w[t] * (layer_scale * branch).  With ``in_w`` returns
+    layernorm(sum_s in_w[s] x_s) of the streams as they then are, in ``out_dtype``: the next sublayer's input.
+    With ``total`` (32-bit ``[tokens, width]``) the sum of the streams is written there."""
+    _gpu(streams, seed, layer_scale, mix, out_w, in_w, norm_w, norm_b, total)
+    _need(streams.dim() == 3 and streams.dtype == torch.float32 and streams.is_contiguous(),
+          "streams_update: contiguous 32-bit streams [S, tokens, width]")
+    S, n, width = streams.shape
+    second, wa, wb = None, 1.0, 0.0
+    if isinstance(branch, BranchSum):
+        branch, second, wa, wb = branch.x, branch.y, branch.a, branch.b
+    bptr, slices, stride, sptr, s_slices, s_stride = None, 0, 0, None, 0, 0
+    if branch is not None:
+        bptr, slices, stride, rows, b_width, bdtype = _branch_args(branch, "streams_update")
+        _need((rows, b_width, bdtype) == (n, width, out_dtype), "streams_update: the branch must match the streams")
+        if not isinstance(branch, SlicedSums):
+            _need(branch.is_contiguous(), "streams_update: a contiguous branch")
+        _need(mix is not None and out_w is not None and mix.shape == (S, S) and out_w.shape == (S,)
+              and mix.dtype == out_w.dtype == torch.float32 and mix.is_contiguous(),
+              "streams_update: 32-bit weights [S, S] and [S] go with a branch")
+        if second is not None:
+            sptr, s_slices, s_stride, s_rows, s_width, s_dtype = _branch_args(second, "streams_update")
+            _need((s_rows, s_width, s_dtype) == (n, width, out_dtype), "streams_update: two branches of one shape and type")
+    _need(seed is None or (seed.shape == (n, width) and seed.dtype == torch.float32 and seed.is_contiguous()),
+          "streams_update: a 32-bit seed of a stream's shape")
+    _need(layer_scale is None or (layer_scale.shape == (width,) and layer_scale.dtype == torch.float32),
+          "streams_update: a 32-bit layer scale of the row's width")
+    _need(total is None or (total.shape == (n, width) and total.dtype == torch.float32 and total.is_contiguous()),
+          "streams_update: a 32-bit total of a stream's shape")
+    nxt = None
+    if in_w is not None:
+        _need(in_w.shape == (S,) and in_w.dtype == torch.float32, "streams_update: 32-bit input weights [S]")
+        _need(norm_w is not None and norm_b is not None and norm_w.shape == (width,) and norm_b.shape == (width,)
+              and norm_w.dtype == norm_b.dtype and norm_w.dtype in _DT, "streams_update: the next norm's weight and bias")
+        nxt = torch.empty((n, width), dtype=out_dtype, device=streams.device)
+    _check(library().rv_streams_update(
+        _stream(), _ptr(streams), _c_ll(n * width), _ptr(seed), bptr, _c_int(slices), _c_ll(stride), sptr,
+        _c_int(s_slices), _c_ll(s_stride), _c_float(wa), _c_float(wb), _ptr(layer_scale), _ptr(mix), _ptr(out_w),
+        _c_float(mult), _ptr(in_w), _ptr(norm_w), _ptr(norm_b),
+        _c_int(norm_w is not None and norm_w.dtype == torch.float32), _ptr(nxt), _ptr(total), _DT[out_dtype], _c_int(S),
+        _c_int(n), _c_int(width), _c_float(eps)))
+    return nxt
+
+
+# ---- a matrix memory with log gates; a gated linear recurrent unit -----------------------------------------------
+def matrix_memory(rows: torch.Tensor, q_col: int, k_col: int, v_col: int, i_col: int, f_col: int, i_bias: torch.Tensor,
+                  f_bias: torch.Tensor, cap: float, q_scale: float, slots: torch.Tensor, s_off: int, n_off: int,
+                  m_off: int, step, heads: int, dk: int, dv: int) -> torch.Tensor:
+    """The matrix memory over the step's tokens, request by request in order.  The rows hold, head after head,
+    queries at ``q_col`` and keys at ``k_col`` (``dk`` a head), values at ``v_col`` (``dv`` a head) and the two
+    gates' inputs at ``i_col + h`` and ``f_col + h``.  Log gates i = cap tanh((a_i + i_bias) / cap),
+    f = logsigmoid(cap tanh((a_f + f_bias) / cap)); m' = max(f + m, i); S' = e^(f + m - m') S + e^(i - m') k v^T, n
+    likewise with k alone; o = S'^T q / (max(|n' . q|, e^(-m')) + 1e-6), q times ``q_scale``.  In the request's
+    32-bit slot S lies at ``s_off`` as ``[heads, dv, dk]``, n at ``n_off`` ``[heads, dk]``, m at ``m_off`` ``[heads]``.
+    Returns o as float32 ``[tokens, heads * dv]``."""
+    _gpu(i_bias, f_bias)
+    n = rows.shape[0]
+    _need(rows.is_cuda and rows.dim() == 2 and rows.stride(1) == 1 and rows.dtype in _DT and n == step.num_tokens,
+          "matrix_memory: rows of the step's tokens")
+    width = rows.shape[1]
+    _need(min(q_col, k_col, v_col, i_col, f_col) >= 0 and max(q_col, k_col) + heads * dk <= width
+          and v_col + heads * dv <= width and max(i_col, f_col) + heads <= width, "matrix_memory: heads outside the rows")
+    _need(i_bias.shape == (heads,) and f_bias.shape == (heads,) and i_bias.dtype == f_bias.dtype == torch.float32,
+          "matrix_memory: float32 gate biases, one a head")
+    stride = _state_args(slots, "matrix_memory")
+    size = slots.shape[1]
+    _need(0 <= s_off and s_off + heads * dk * dv <= size and 0 <= n_off and n_off + heads * dk <= size
+          and 0 <= m_off and m_off + heads <= size, "matrix_memory: the state lies outside the slot")
+    gates = torch.empty((n, heads, 3), dtype=torch.float32, device=rows.device)
+    out = torch.empty((n, heads * dv), dtype=torch.float32, device=rows.device)
+    lib = library()
+    _check(lib.rv_memory_gates(
+        _stream(), _ptr(rows), _dt(rows), _c_ll(rows.stride(0)), _c_int(q_col), _c_int(k_col), _c_int(i_col),
+        _c_int(f_col), _ptr(i_bias), _ptr(f_bias), _c_float(cap), _c_float(q_scale), _ptr(slots), _c_ll(stride),
+        _c_ll(n_off), _c_ll(m_off), _ptr(step.q_start), _ptr(step.state_slot), _ptr(gates), _c_int(step.num_requests),
+        _c_int(heads), _c_int(dk)))
+    _check(lib.rv_memory_matrix(
+        _stream(), _ptr(rows), _dt(rows), _c_ll(rows.stride(0)), _c_int(q_col), _c_int(k_col), _c_int(v_col),
+        _c_float(q_scale), _ptr(gates), _ptr(slots), _c_ll(stride), _c_ll(s_off), _ptr(step.q_start),
+        _ptr(step.state_slot), _ptr(out), _c_int(step.num_requests), _c_int(heads), _c_int(dk), _c_int(dv),
+        _c_int(step.max_portion)))
+    return out
+
+
+def gated_linear_scan(u: torch.Tensor, gates: torch.Tensor, block: int, r_bias: torch.Tensor, i_bias: torch.Tensor,
+                      lam: torch.Tensor, y: torch.Tensor, y_col0: int, slots: torch.Tensor, s_off: int,
+                      step) -> torch.Tensor:
+    """The gated linear recurrent unit over the step's tokens, request by request in order, a channel at a time:
+    r = sigmoid(g_r + r_bias), i = sigmoid(g_i + i_bias), log a = -8 r softplus(lam), S' = a S + sqrt(1 - a^2) i u,
+    out = S' * gelu_tanh(y).  ``u [tokens, channels]`` is the convolved input, ``gates`` float32
+    ``[tokens, 2 channels]`` holds for block b of ``block`` channels its g_r and then its g_i, ``y`` the other
+    branch before its activation at ``y_col0`` of its rows.  S is 32-bit at ``s_off`` of the request's slot."""
+    _gpu(u, gates, r_bias, i_bias, lam)
+    n, channels = u.shape
+    _need(n == step.num_tokens and u.dtype in _DT and u.stride(1) == 1, "gated_linear_scan: rows of the step's tokens")
+    _need(gates.shape == (n, 2 * channels) and gates.dtype == torch.float32 and gates.stride(1) == 1,
+          "gated_linear_scan: float32 gates [tokens, 2 channels]")
+    _need(channels % block == 0, "gated_linear_scan: blocks of equal size")
+    for t in (r_bias, i_bias, lam):
+        _need(t.shape == (channels,) and t.dtype == torch.float32, "gated_linear_scan: float32 biases and rates, one a channel")
+    _need(y.is_cuda and y.dim() == 2 and y.stride(1) == 1 and y.dtype == u.dtype and y.shape[0] == n
+          and 0 <= y_col0 and y_col0 + channels <= y.shape[1], "gated_linear_scan: the other branch lies outside its rows")
+    stride = _state_args(slots, "gated_linear_scan")
+    _need(0 <= s_off and s_off + channels <= slots.shape[1], "gated_linear_scan: the state lies outside the slot")
+    out = torch.empty((n, channels), dtype=u.dtype, device=u.device)
+    _check(library().rv_gated_linear_scan(
+        _stream(), _ptr(u), _c_ll(u.stride(0)), _ptr(gates), _c_ll(gates.stride(0)), _c_int(block), _ptr(r_bias),
+        _ptr(i_bias), _ptr(lam), y.data_ptr() + y_col0 * y.element_size(), _c_ll(y.stride(0)), _ptr(slots),
+        _c_ll(stride), _c_ll(s_off), _ptr(step.q_start), _ptr(step.state_slot), _ptr(out), _dt(u),
+        _c_int(step.num_requests), _c_int(channels), _c_int(step.max_portion)))
+    return out
+
+
+def gemm_blocks_f32(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """A block-diagonal product with 32-bit results: ``w`` is ``[blocks, N, K]``; block b multiplies columns
+    ``b K .. + K`` of the rows of ``a`` and fills columns ``b N .. + N`` of the float32 ``[rows, blocks N]``."""
+    _need(a.is_cuda and w.is_cuda and a.dim() == 2 and w.dim() == 3 and w.is_contiguous() and a.stride(1) == 1
+          and a.dtype == w.dtype and a.dtype in _DT, "gemm_blocks_f32: rows and [blocks, N, K] matrices of one type")
+    blocks, n, k = w.shape
+    m = a.shape[0]
+    _need(blocks * k == a.shape[1], "gemm_blocks_f32: the blocks' inputs fill the rows")
+    out = torch.empty((m, blocks * n), dtype=torch.float32, device=a.device)
+    _check(library().rv_gemm_groups_plain(
+        _stream(), _ptr(a), _dt(a), _ptr(w), _dt(w), _ptr(out), _dt(out), None, None, _c_int(blocks), _c_int(m),
+        _c_int(n), _c_int(k), _c_ll(a.stride(0)), _c_ll(k), _c_ll(out.stride(0)), _c_ll(k), _c_ll(n * k), _c_ll(n),
+        None, _c_ll(0)))
+    return out
+
+
+# ---- experts chosen by a learned router ---------------------------------------------------------------------------
+MOE_MAX_EXPERTS_TOPK = 1024
+
+
+def moe_topk(logits: torch.Tensor, top: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """For every row of the float32 router logits ``[tokens, experts]`` its ``top`` largest (the largest first; of
+    equal ones the lower index): (chosen int32 ``[tokens, top]``, weights float32 ``[tokens, top]`` =
+    sigmoid(logit))."""
+    _gpu(logits)
+    _need(logits.dim() == 2 and logits.dtype == torch.float32 and logits.is_contiguous(), "moe_topk: float32 logits")
+    n, experts = logits.shape
+    _need(1 <= top <= experts, f"moe_topk: {top} of {experts} experts")
+    chosen = torch.empty((n, top), dtype=torch.int32, device=logits.device)
+    weights = torch.empty((n, top), dtype=torch.float32, device=logits.device)
+    _check(library().rv_moe_topk(_stream(), _ptr(logits), _c_int(n), _c_int(experts), _c_int(top), _ptr(chosen),
+                                 _ptr(weights)))
+    return chosen, weights
+
+
+def moe_scale_rows(x: torch.Tensor, slot_of: torch.Tensor, weights: torch.Tensor, top: int, capacity: int) -> torch.Tensor:
+    """The sorted rows of the experts' first product where a choice's weight multiplies the expert's input:
+    xs[slot_of[t * top + k]] = weights[t, k] * x[t]; filling rows are zeros."""
+    _gpu(x, slot_of, weights)
+    _i32(slot_of)
+    n, width = x.shape
+    _need(x.is_contiguous() and x.dtype in _DT and slot_of.numel() == n * top and weights.numel() == n * top
+          and weights.dtype == torch.float32, "moe_scale_rows: one weight and one sorted row for every choice")
+    xs = torch.zeros((capacity, width), dtype=x.dtype, device=x.device)
+    _check(library().rv_moe_scale_rows(_stream(), _ptr(x), _ptr(slot_of), _ptr(weights), _c_int(top), _ptr(xs), _dt(x),
+                                       _c_int(n), _c_int(width)))
+    return xs

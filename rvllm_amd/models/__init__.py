@@ -1,6 +1,6 @@
 """Architectures.  Importing the package registers the ones the framework ships."""
 
-from . import gemma3, pinorax, rufedra  # noqa: F401  (register themselves)
+from . import dafalix, gemma3, pinorax, rufedra  # noqa: F401  (register themselves)
 from .model import DecoderModel
 from .registry import (Architecture, architecture_names, architecture_of, get_architecture, load_config,
                        register_architecture, unregister_architecture)

@@ -28,6 +28,12 @@ class DecoderModel:
         self.head = HEADS.build(spec.head, hidden_size=H, vocab_size=V, embedding=self.embedding)
         self.device: Optional[torch.device] = None
         self.dtype: Optional[torch.dtype] = None
+        # Where each run's cache lies in the list of caches: a layer's own (copy 0) at the layer's index, as the
+        # storage and the tests address it; the further copies of layers that run several times follow the layers.
+        self.cache_index: dict[tuple[int, int], int] = {(i, 0): i for i in range(len(spec.layers))}
+        for entry in spec.schedule:
+            if entry.cache_from is None and (entry.layer, entry.copy) not in self.cache_index:
+                self.cache_index[(entry.layer, entry.copy)] = len(self.cache_index)
 
     # ---- weights -----------------------------------------------------
     def param_specs(self) -> list[ParamSpec]:
@@ -95,16 +101,22 @@ class DecoderModel:
 
     # ---- cache needs ---------------------------------------------------
     def cache_needs(self) -> list:
-        """For every layer what its mixer keeps between steps (or None for a
-        layer that only ever reads another layer's cache)."""
-        owners = {e.layer for e in self.spec.schedule if e.cache_from is None}
-        return [block.mixer.cache_need() if i in owners else None for i, block in enumerate(self.blocks)]
+        """For every cache what its layer's mixer keeps between steps (or None for a
+        layer that only ever reads another layer's cache): one entry a layer, then one for
+        every further copy of a layer that runs several times with a cache each (``cache_index``)."""
+        owners = {(e.layer, e.copy) for e in self.spec.schedule if e.cache_from is None}
+        needs = [None] * len(self.cache_index)
+        for (layer, copy), at in self.cache_index.items():
+            if (layer, copy) in owners:
+                needs[at] = self.blocks[layer].mixer.cache_need()
+        return needs
 
     # ---- run ---------------------------------------------------------
     def forward(self, step, caches: list) -> torch.Tensor:
         """Runs the step's tokens; returns float32 logits ``[wanted rows, vocab]``.
 
-        ``caches[i]`` is the cache view of layer i."""
+        ``caches[i]`` is the cache view of layer i (``cache_index`` for the copies of a layer that runs
+        several times)."""
         x = torch.empty((step.num_tokens, self.spec.hidden_size), device=self.device,
                         dtype=torch.float32 if self.spec.residual_float32 else self.dtype)
         self.embedding.forward(step, x)
@@ -112,7 +124,8 @@ class DecoderModel:
         entered = None
         for i, entry in enumerate(schedule):
             block = self.blocks[entry.layer]
-            cache = caches[entry.layer] if entry.cache_from is None else reader_view(caches[entry.cache_from])
+            cache = (caches[self.cache_index[(entry.layer, entry.copy)]] if entry.cache_from is None
+                     else reader_view(caches[entry.cache_from]))
             nxt = self.blocks[schedule[i + 1].layer].entry_norm() if i + 1 < len(schedule) else None
             # None means the block did not apply the next entry norm; the next block then does
             entered = block.forward(x, step, cache, entered=entered, then=nxt)

@@ -13,6 +13,10 @@ activations in bf16, the norm reads the one and writes the other.
 y = x * rsqrt(mean(x^2) + eps) * g.  Its input may be a residual stream that a
 bf16 model keeps in 32 bits; the output has the activations' type.  ``suffix``
 is what the tensor's name is followed by (``.weight`` if absent).
+
+``layernorm``: y = (x - mean) / sqrt(mean((x - mean)^2) + eps) * weight + bias, all in 32-bit.  ``suffix`` follows
+the weight's name (``.weight`` if absent) and ``bias_suffix`` the bias's (``.bias`` if absent).  Reads a 32-bit
+stream or the activations' type, writes the activations' type.
 """
 
 from __future__ import annotations
@@ -101,5 +105,35 @@ class ScalarRMSNorm(Norm):
         return ops.scalar_rmsnorm(x, self.gain, self.eps, self.out_dtype, rows=rows)
 
 
+class LayerNorm(Norm):
+    def __init__(self, spec: PartSpec, *, width: int, name: str):
+        self.width = int(width)
+        self.name = name
+        self.eps = float(spec["eps"])
+        self.suffix = str(spec.get("suffix", ".weight"))
+        self.bias_suffix = str(spec.get("bias_suffix", ".bias"))
+        self.weight: Optional[torch.Tensor] = None
+        self.bias: Optional[torch.Tensor] = None
+        self.out_dtype: Optional[torch.dtype] = None
+
+    def param_specs(self, prefix: str) -> list[ParamSpec]:
+        at = tensor_path(prefix, self.name)
+        return [ParamSpec(at + self.suffix, (self.width,), init=("normal_about", 1.0, 0.1)),
+                ParamSpec(at + self.bias_suffix, (self.width,), init=("normal", 0.1))]
+
+    def bind(self, tensors, prefix, device, dtype) -> None:
+        at = tensor_path(prefix, self.name)
+        self.weight = tensors[at + self.suffix].to(device=device, dtype=torch.float32).contiguous()
+        self.bias = tensors[at + self.bias_suffix].to(device=device, dtype=torch.float32).contiguous()
+        self.out_dtype = dtype
+
+    def forward(self, x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return ops.layernorm(x, self.weight, self.bias, self.eps, self.out_dtype, out=out)
+
+    def forward_rows(self, x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
+        return ops.layernorm(x, self.weight, self.bias, self.eps, self.out_dtype, rows=rows)
+
+
 NORMS.register("rmsnorm", RMSNorm)
+NORMS.register("layernorm", LayerNorm)
 NORMS.register("rmsnorm_scalar", ScalarRMSNorm)

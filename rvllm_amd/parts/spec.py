@@ -50,10 +50,14 @@ class LayerSpec:
 @dataclasses.dataclass(frozen=True)
 class ScheduleEntry:
     """One run of a layer.  ``cache_from`` names the layer whose cache this
-    run reads instead of keeping one of its own."""
+    run reads instead of keeping one of its own.  ``copy`` tells the layer's
+    caches apart where it runs several times in a step with the same weights
+    and every run keeps keys or a state of its own (a stretch of layers that is
+    walked more than once): runs with the same ``copy`` share one cache."""
 
     layer: int
     cache_from: Optional[int] = None
+    copy: int = 0
 
 
 @dataclasses.dataclass(frozen=True)
@@ -79,7 +83,9 @@ class ModelSpec:
         for entry in self.schedule:
             if not 0 <= entry.layer < n:
                 raise ValueError(f"schedule names layer {entry.layer}, model has {n}")
-            if entry.cache_from is None:
+            if entry.copy < 0 or (entry.copy and entry.cache_from is not None):
+                raise ValueError(f"layer {entry.layer}: a run has a cache of its own (copy >= 0) or reads another's")
+            if entry.cache_from is None and entry.copy == 0:
                 owners.add(entry.layer)
         for entry in self.schedule:
             if entry.cache_from is not None and entry.cache_from not in owners:
