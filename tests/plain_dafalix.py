@@ -198,10 +198,14 @@ def recurrent_unit_mixer(h, W, p, m):
 
 
 # ---- experts -----------------------------------------------------------------------
-def routed_experts(h, W, p, mlp):
-    """Scores sigmoid(W_router h); the ``top`` largest choose the experts; an expert's input is score * h."""
+def routed_experts(h, W, p, mlp, margins=None):
+    """Scores sigmoid(W_router h); the ``top`` largest choose the experts; an expert's input is score * h.
+    ``margins`` collects, for every token, by how much the last chosen logit leads the first one left out."""
     E, top = mlp["router"]["experts"], mlp["router"]["top"]
     scores = torch.sigmoid(r(h) @ W[p + "router"].T)
+    if margins is not None:
+        z = torch.sort(r(h) @ W[p + "router"].T, dim=-1, descending=True).values
+        margins.append(z[:, top - 1] - z[:, top] if top < E else torch.full((h.shape[0],), float("inf"), dtype=F))
     chosen = torch.topk(scores, top, dim=-1).indices
     out = torch.zeros(h.shape[0], W[p + "e0.down"].shape[0], dtype=F)
     for t in range(h.shape[0]):
@@ -228,8 +232,9 @@ def layer_runs(cfg) -> list[int]:
     return list(range(loop["start"])) + inside * loop["times"] + list(range(loop["stop"], n))
 
 
-def forward(W, cfg, ids, streams=None):
-    """Logits [T, vocab] of one sequence; ``streams`` collects the summed residual streams after every layer run."""
+def forward(W, cfg, ids, streams=None, margins=None):
+    """Logits [T, vocab] of one sequence; ``streams`` collects the summed residual streams after every layer run,
+    ``margins`` the routers' leads (``routed_experts``), one entry for every run of a layer with experts."""
     eps = cfg["norm"]["eps"]
     mult, S = cfg["residual_mult"], cfg["streams"]
     xs = [W["embed"][torch.tensor(ids, dtype=torch.long)].clone() for _ in range(S)]
@@ -241,7 +246,7 @@ def forward(W, cfg, ids, streams=None):
             hc = p + f"hc{q}."
             u = sum(W[hc + "in"][s] * xs[s] for s in range(S))
             h = r(layer_norm(u, eps, W[p + f"norm{q}"], W[p + f"norm{q}.b"]))
-            y = mixer(h, W, p, layer, eps) if sub == "mixer" else routed_experts(h, W, p + "mlp.", layer["mlp"])
+            y = mixer(h, W, p, layer, eps) if sub == "mixer" else routed_experts(h, W, p + "mlp.", layer["mlp"], margins)
             y = y * W[p + f"ls{q}"]
             xs = [sum(W[hc + "mix"][s, t] * xs[s] for s in range(S)) + mult * W[hc + "out"][t] * y for t in range(S)]
         if streams is not None:
@@ -256,6 +261,16 @@ def rounding_error(W, cfg, ids, exact=None):
     with rounded():
         coarse = forward(W, cfg, ids)
     return (coarse - exact).abs().max(-1).values
+
+
+def close_calls(W, cfg, ids, lead=0.2):
+    """For every position whether some router chose there by less than ``lead``: 16-bit rounding of the router's
+    input may then choose another expert, and every later position of the sequence may hear of it."""
+    margins = []
+    forward(W, cfg, ids, margins=margins)
+    if not margins:
+        return torch.zeros(len(ids), dtype=torch.bool)
+    return torch.stack(margins).min(0).values < lead
 
 
 def greedy(W, cfg, prompt, count):
