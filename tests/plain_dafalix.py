@@ -198,15 +198,26 @@ def recurrent_unit_mixer(h, W, p, m):
 
 
 # ---- experts -----------------------------------------------------------------------
-def routed_experts(h, W, p, mlp, margins=None):
+def routed_experts(h, W, p, mlp, margins=None, forced=None, lead=0.2):
     """Scores sigmoid(W_router h); the ``top`` largest choose the experts; an expert's input is score * h.
-    ``margins`` collects, for every token, by how much the last chosen logit leads the first one left out."""
+    ``margins`` collects, for every token, by how much the last chosen logit leads the first one left out.
+    ``forced`` [T, top] gives the experts instead (what an engine chose): each must be one of the largest or fall
+    short of them by less than ``lead``, the room that rounding has, but for one token in fifty (or one), whose
+    router may have got an input that an ill-conditioned read-out before it moved far; everything else is computed
+    as ever."""
     E, top = mlp["router"]["experts"], mlp["router"]["top"]
     scores = torch.sigmoid(r(h) @ W[p + "router"].T)
     if margins is not None:
         z = torch.sort(r(h) @ W[p + "router"].T, dim=-1, descending=True).values
         margins.append(z[:, top - 1] - z[:, top] if top < E else torch.full((h.shape[0],), float("inf"), dtype=F))
     chosen = torch.topk(scores, top, dim=-1).indices
+    if forced is not None:
+        z = r(h) @ W[p + "router"].T
+        chosen = torch.as_tensor(forced, dtype=torch.long)
+        assert chosen.shape == (h.shape[0], top) and all(len(set(row)) == top for row in chosen.tolist())
+        short = torch.sort(z, dim=-1, descending=True).values[:, top - 1:top] - z.gather(1, chosen)
+        far = int((short.max(-1).values >= lead).sum())
+        assert far <= max(1, h.shape[0] // 50), f"{far} of {h.shape[0]} tokens chose an expert far from the largest"
     out = torch.zeros(h.shape[0], W[p + "e0.down"].shape[0], dtype=F)
     for t in range(h.shape[0]):
         for e in chosen[t].tolist():
@@ -232,9 +243,11 @@ def layer_runs(cfg) -> list[int]:
     return list(range(loop["start"])) + inside * loop["times"] + list(range(loop["stop"], n))
 
 
-def forward(W, cfg, ids, streams=None, margins=None):
+def forward(W, cfg, ids, streams=None, margins=None, forced=None):
     """Logits [T, vocab] of one sequence; ``streams`` collects the summed residual streams after every layer run,
-    ``margins`` the routers' leads (``routed_experts``), one entry for every run of a layer with experts."""
+    ``margins`` the routers' leads (``routed_experts``), one entry for every run of a layer with experts;
+    ``forced`` gives the experts of every such run, in their order."""
+    forced = None if forced is None else list(forced)
     eps = cfg["norm"]["eps"]
     mult, S = cfg["residual_mult"], cfg["streams"]
     xs = [W["embed"][torch.tensor(ids, dtype=torch.long)].clone() for _ in range(S)]
@@ -246,7 +259,8 @@ def forward(W, cfg, ids, streams=None, margins=None):
             hc = p + f"hc{q}."
             u = sum(W[hc + "in"][s] * xs[s] for s in range(S))
             h = r(layer_norm(u, eps, W[p + f"norm{q}"], W[p + f"norm{q}.b"]))
-            y = mixer(h, W, p, layer, eps) if sub == "mixer" else routed_experts(h, W, p + "mlp.", layer["mlp"], margins)
+            y = mixer(h, W, p, layer, eps) if sub == "mixer" else routed_experts(
+                h, W, p + "mlp.", layer["mlp"], margins, None if forced is None else forced.pop(0))
             y = y * W[p + f"ls{q}"]
             xs = [sum(W[hc + "mix"][s, t] * xs[s] for s in range(S)) + mult * W[hc + "out"][t] * y for t in range(S)]
         if streams is not None:
@@ -255,12 +269,25 @@ def forward(W, cfg, ids, streams=None, margins=None):
     return r(layer_norm(x, eps, W["final.norm"], W["final.norm.b"])) @ W["embed"].T
 
 
-def rounding_error(W, cfg, ids, exact=None):
+def rounding_error(W, cfg, ids, exact=None, forced=None):
     """For every position, the largest difference that rounding alone (``rounded``) makes to a logit."""
-    exact = forward(W, cfg, ids) if exact is None else exact
+    exact = forward(W, cfg, ids, forced=forced) if exact is None else exact
     with rounded():
-        coarse = forward(W, cfg, ids)
+        coarse = forward(W, cfg, ids, forced=forced)
     return (coarse - exact).abs().max(-1).values
+
+
+def float32_error(W, cfg, ids, exact, forced=None):
+    """For every position, the largest difference to ``exact`` of this same implementation run in 32-bit throughout:
+    what 32-bit arithmetic alone costs there (a read-out that all but cancels, a norm that blows a remainder up)."""
+    global F
+    F = torch.float32
+    try:
+        W32 = {k: (v.float() if v.is_floating_point() else v) for k, v in W.items()}
+        got = forward(W32, cfg, ids, forced=forced).double()
+    finally:
+        F = torch.float64
+    return (got - exact).abs().max(-1).values
 
 
 def close_calls(W, cfg, ids, lead=0.2):

@@ -4,11 +4,12 @@ with experts or none, a looped stretch anywhere or none, 1-5 streams; matrix mem
 that are equal or not, windows of 1-150, rotations of none, a part or all of a head with any base and factor;
 recurrent units of 8-200 channels in 1 to as many blocks, 1-5 taps; 1-20 experts of which 1 to all are chosen;
 sequences of 1-260 tokens under the four cuttings, pages of 16 / 32 / 64, both dtypes.  Either dtype is held to the
-larger of its flat share of the largest logit and three times the error that rounding alone causes at the position
-(``plain_dafalix.rounding_error``, measured with bf16's roundings; a 32-bit engine rounds 65 536 times finer but at
-every operation, counted as twice as often).  Where a router's choice hangs on less than 16-bit rounding moves it,
-the bf16 engine may choose another expert: from the first such position of a sequence on, a tenth of the positions
-may be over (``trace_tools.compare_where_routers_may_differ``).  A few seeds are committed; ``draw`` serves a longer run by hand."""
+larger of its flat share of the largest logit and three times the error that its rounding alone causes at the position
+in the plain implementation (``plain_dafalix.rounding_error`` with bf16's roundings, ``float32_error`` for a run in
+32-bit throughout: a matrix memory's read-out can all but cancel, and the norm behind it blows the remainder up).
+Where a router's choice hangs on less than rounding moves it, the engine may choose another expert: its choices are
+recorded, checked to be such close calls, and given to the plain implementation, so that every position is held to
+the same measure.  A few seeds are committed; ``draw`` serves a longer run by hand."""
 
 import json
 import random
@@ -37,7 +38,7 @@ def draw(seed: int) -> dict:
             return None
         experts = rng.choice([1, 2, 3, 5, 8, 12, 20])
         return {"kind": "moe", "expert": {"ff": size(8, 120)},
-                "router": {"experts": experts, "top": rng.choice([1, 1, 2, experts, rng.randint(1, experts)])}}
+                "router": {"experts": experts, "top": min(experts, rng.choice([1, 1, 2, experts, rng.randint(1, experts)]))}}
 
     layers = []
     for _ in range(rng.randint(1, 5)):
@@ -70,7 +71,7 @@ def draw(seed: int) -> dict:
     return doc
 
 
-@pytest.mark.parametrize("seed", [1, 2, 3, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("seed", [3, 7, 12, 19, 40, 46, 51, 65])
 def test_a_configuration_drawn_at_random(tmp_path, seed):
     doc = draw(seed)
     tiny_dafalix.CONFIGS["random"] = (doc, seed)
@@ -82,9 +83,7 @@ def test_a_configuration_drawn_at_random(tmp_path, seed):
     rng = random.Random(seed + 1000)
     lengths = [rng.choice([1, 2, 15, 16, 17, 33]), rng.randint(3, 120), rng.randint(100, 260)]
     seqs = tt.make_sequences(cfg["vocab"], lengths, seed=seed)
-    refs = {rid: PD.forward(weights, cfg, ids) for rid, ids in seqs.items()}
-    rounding = {rid: PD.rounding_error(weights, cfg, ids, refs[rid]).numpy() for rid, ids in seqs.items()}
-    calls = {rid: PD.close_calls(weights, cfg, ids).numpy() for rid, ids in seqs.items()}
+    measured: dict = {}
     page_size = rng.choice([16, 32, 64])
     for dtype in ("float32", "bfloat16"):
         for mode, make in (("whole", tt.trace_whole), ("tail", tt.trace_tail), ("portions", tt.trace_portions),
@@ -93,18 +92,22 @@ def test_a_configuration_drawn_at_random(tmp_path, seed):
             most = max(tt.required_tokens(steps), page_size)
             runner = ModelRunner.from_model_dir(folder, EngineConfig(
                 dtype=dtype, page_size=page_size, max_model_len=most, max_num_seqs=4, max_num_batched_tokens=most,
-                max_prefill_chunk=most, max_cache_tokens=most))
-            got = tt.collect(steps, tt.run_in_process(runner, steps), cfg["vocab"])
+                max_prefill_chunk=most, max_cache_tokens=most, use_graphs=dtype != "bfloat16"))
+            with tt.RecordedChoices() as choices:
+                got = tt.collect(steps, tt.run_in_process(runner, steps, choices), cfg["vocab"])
+            forced = choices.by_request(steps)
             prefix = steps[0]["entries"][0]["id"].split("-")[0]
-            for name, ref in refs.items():
+            for name, ids in seqs.items():
                 what = f"seed {seed} {dtype} {mode} {name}: {json.dumps(doc)}"
-                arr = np.asarray(got[f"{prefix}-{name}"], dtype=np.float64)
-                assert arr.shape == tuple(ref.shape) and np.isfinite(arr).all(), what
-                err = np.abs(arr - ref.numpy()).max(-1)
-                finer = 1.0 if dtype == "bfloat16" else 2.0 ** -15
-                allowed = np.maximum(tt.TOLERANCE[dtype] * float(ref.abs().max()), 3.0 * finer * rounding[name])
-                if dtype == "bfloat16":
-                    tt.compare_where_routers_may_differ(arr, ref, allowed, calls[name], what)
-                    continue
-                worst = int((err / allowed).argmax())
-                assert err[worst] <= allowed[worst], f"position {worst}: {err[worst]:.3e} > {allowed[worst]:.3e}; {what}"
+                # against the plain implementation with the experts that the engine chose (each a close call or the
+                # plain choice); the allowance is three times what the dtype's rounding alone does at the position
+                chosen = forced.get(f"{prefix}-{name}") or []
+                key = (name, dtype, b"".join(c.tobytes() for c in chosen))
+                if key not in measured:  # the cuttings mostly choose alike
+                    ref = PD.forward(weights, cfg, ids, forced=chosen)
+                    noise = (PD.rounding_error(weights, cfg, ids, ref, forced=chosen) if dtype == "bfloat16"
+                             else PD.float32_error(weights, cfg, ids, ref, forced=chosen)).numpy()
+                    measured[key] = (ref, noise)
+                ref, noise = measured[key]
+                allowed = np.maximum(tt.TOLERANCE[dtype] * float(ref.abs().max()), 3.0 * noise)
+                tt.held_to_rounding(got[f"{prefix}-{name}"], ref, allowed, what)

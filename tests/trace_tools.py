@@ -131,7 +131,46 @@ def collect(steps, outputs: dict, vocab: int) -> dict[str, np.ndarray]:
     return {rid: np.concatenate(parts) for rid, parts in by_request.items()}
 
 
-def run_in_process(runner, steps) -> dict[int, np.ndarray]:
+class RecordedChoices:
+    """While open, keeps what every call of the engine's router kernel chose (``ops.moe_topk``), call by call.
+    ``by_request(steps)`` sorts it by request: for every run of a layer with experts, in the order of the runs, the
+    experts of the request's tokens ``[tokens, top]``.  Steps replayed from a recorded graph call nothing: the
+    engine is to run without graphs meanwhile."""
+
+    def __enter__(self):
+        from rvllm_amd.kernels import ops
+
+        self.ops, self.inner, self.calls, self.per_step = ops, ops.moe_topk, [], []
+
+        def recording(logits, top):
+            chosen, weights = self.inner(logits, top)
+            self.calls.append(chosen.cpu().numpy().copy())
+            return chosen, weights
+
+        ops.moe_topk = recording
+        return self
+
+    def __exit__(self, *exc):
+        self.ops.moe_topk = self.inner
+
+    def end_step(self):
+        self.per_step.append(self.calls)
+        self.calls = []
+
+    def by_request(self, steps) -> dict:
+        out: dict = {}
+        for st, calls in zip(steps, self.per_step):
+            row = 0
+            for e in st["entries"]:
+                n = len(e["tokens"])
+                runs = out.setdefault(e["id"], [[] for _ in calls])
+                for run, chosen in zip(runs, calls):
+                    run.append(chosen[row:row + n])
+                row += n
+        return {rid: [np.concatenate(run) for run in runs] for rid, runs in out.items()}
+
+
+def run_in_process(runner, steps, choices: "RecordedChoices | None" = None) -> dict[int, np.ndarray]:
     outputs = {}
     for st in steps:
         entries = []
@@ -142,6 +181,8 @@ def run_in_process(runner, steps) -> dict[int, np.ndarray]:
         logits = runner.step(entries)
         if logits.shape[0]:
             outputs[st["step"]] = logits.float().cpu().numpy()
+        if choices is not None:
+            choices.end_step()
         for rid in st["end"]:
             runner.release(rid)
         runner.cache.check()
@@ -210,3 +251,15 @@ def compare_where_routers_may_differ(got, want, allowed, close, what: str = "") 
                                     f"{err[int(np.argmax(over[:first]))]:.3e} before any router's close call (at {first})")
     assert int(over[first:].sum()) <= max(2, (len(over) - first) // 10), (
         f"{what}: {int(over[first:].sum())} of {len(over) - first} positions over after the first close call")
+
+
+def held_to_rounding(got, want, allowed, what: str = "") -> None:
+    """Every position within one and a half times ``allowed`` (itself three times what one run's rounding did at
+    the position), and at most one position in fifty (or one) over ``allowed``."""
+    got = np.asarray(got, dtype=np.float64)
+    want = want.detach().double().numpy() if hasattr(want, "detach") else np.asarray(want, dtype=np.float64)
+    assert got.shape == want.shape and np.isfinite(got).all(), what
+    ratio = np.abs(got - want).max(-1) / allowed
+    worst = int(ratio.argmax())
+    assert ratio[worst] <= 1.5, f"{what}: position {worst} is at {ratio[worst]:.2f} of its allowance {allowed[worst]:.3e}"
+    assert int((ratio > 1.0).sum()) <= max(1, len(ratio) // 50), f"{what}: {int((ratio > 1.0).sum())} of {len(ratio)} positions over"
