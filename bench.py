@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 8192] [--layers L]
     python bench.py --workload 12b|27b [--requests N] [--layers L]     (another measurement, see WORKLOADS)
-    python bench.py --design pinorax|rufedra [--size s|l] [--layers L]  (another measurement, see DESIGN_SIZES)
+    python bench.py --design pinorax|rufedra|dafalix [--size s|l] [--layers L]  (another measurement, see DESIGN_SIZES)
 
 Default run: the layer sizes of the 4B-sized configuration (34 layers, 5
 sliding : 1 global, hidden 2560, 8 query / 4 key-value heads of 256, GeGLU
@@ -347,6 +347,39 @@ RUFEDRA_SIZES = {
 }
 
 
+# The Dafalix layers: in turn a matrix-memory layer without a feed-forward (``heads`` heads of ``dim``) and a layer with
+# two mixers side by side, attention over a sliding window (half of a head rotated, queries and keys normed) beside a
+# gated linear recurrent unit (``inner`` channels in ``blocks`` blocks), with ``top`` of ``experts`` experts that are
+# together as wide as the dense feed-forward beside them; ``streams`` copies of the residual stream.  Beside it Rufedra,
+# the framework's closest design, at equal size: its delta-rule layer for the matrix memory, its selective scan for
+# the recurrent unit, its dense feed-forward for the experts.
+DAFALIX_SIZES = {
+    "s": dict(RUFEDRA_SIZES["s"], blocks=16, experts=32, top=2, streams=2, gate_cap=15.0),
+    "l": dict(RUFEDRA_SIZES["l"], blocks=16, experts=64, top=4, streams=2, gate_cap=15.0),
+}
+
+
+def dafalix_configs(size: dict, layers: int, positions: int):
+    from rvllm_amd.config.dafalix import DafalixConfig
+
+    memory = {"type": "mlstm", "mlp": None, "mixer": {"heads": size["heads"], "dim": size["dim"], "vdim": size["dim"],
+                                                      "gate_cap": size["gate_cap"]}}
+    left = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["dim"],
+            "scale": size["dim"] ** -0.5, "mask": {"size": size["window"]},
+            "rot": {"dims": size["dim"] // 2, "base": 10000.0, "scaling": {"factor": 1.0}}}
+    right = {"width": size["inner"], "blocks": size["blocks"], "conv": size["conv"]}
+    moe = {"kind": "moe", "expert": {"ff": size["ff"] // size["top"]},
+           "router": {"experts": size["experts"], "top": size["top"]}}
+    parallel = {"type": "parallel", "mlp": moe,
+                "mixer": {"left": left, "right": right, "left_scale": 1.0, "right_scale": 1.0}}
+    dafalix = DafalixConfig.from_dict({
+        "architecture": "Dafalix", "vocab": size["vocab"], "width": size["width"], "norm": {"eps": 1e-6},
+        "residual_mult": 1.0, "streams": size["streams"],
+        "layers": [memory if i % 2 == 0 else parallel for i in range(layers)],
+    }, "bench configuration")
+    return dafalix, rufedra_configs(size, layers, positions)[0]
+
+
 def rufedra_configs(size: dict, layers: int, positions: int):
     from rvllm_amd.config.gemma3 import Gemma3Config
     from rvllm_amd.config.rufedra import RufedraConfig
@@ -405,18 +438,20 @@ def run_design(args) -> int:
     import rvllm_amd.models  # noqa: F401
 
     design = args.design
-    size = (RUFEDRA_SIZES if design == "rufedra" else DESIGN_SIZES)[args.size]
-    make_configs = rufedra_configs if design == "rufedra" else design_configs
+    size = {"rufedra": RUFEDRA_SIZES, "dafalix": DAFALIX_SIZES}.get(design, DESIGN_SIZES)[args.size]
+    make_configs = {"rufedra": rufedra_configs, "dafalix": dafalix_configs}.get(design, design_configs)
+    beside = "rufedra" if design == "dafalix" else "dense"  # the closest design of the framework, at equal size
     layers = args.layers if args.layers != FULL_LAYERS else 8
     context, T = args.context, args.prefill_tokens
     batches = [b for b in (8, 64) if not (args.no_points and b != 8)]
     steps_total = args.steps + args.warmup + 8
     positions = max(context + steps_total + 16, T)
-    out = {"metric": f"prefill and decode of {design.capitalize()} beside the dense decoder, size {args.size}", "unit": "ms",
+    out = {"metric": f"prefill and decode of {design.capitalize()} beside "
+                     f"{'the dense decoder' if beside == 'dense' else beside.capitalize()}, size {args.size}", "unit": "ms",
            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic: random weights, caches filled "
            "with random values, uniform token ids", "config": dict(size, layers=layers, context=context, prefill_tokens=T),
            "designs": {}}
-    for name, cfg in zip((design, "dense"), make_configs(size, layers, positions)):
+    for name, cfg in zip((design, beside), make_configs(size, layers, positions)):
         engine_cfg = EngineConfig(dtype=args.dtype, page_size=args.page_size, max_model_len=positions,
                                   max_num_seqs=max(batches), max_num_batched_tokens=max(T, max(batches)),
                                   max_prefill_chunk=T, max_cache_tokens=max(batches) * (context + steps_total + 16),
@@ -441,8 +476,8 @@ def run_design(args) -> int:
         import gc
         gc.collect()
         torch.cuda.empty_cache()
-    p, d = out["designs"][design], out["designs"]["dense"]
-    out[f"{design}_over_dense"] = {k: round(p[k] / d[k], 3) for k in p if k.endswith("_ms") and k in d}
+    p, d = out["designs"][design], out["designs"][beside]
+    out[f"{design}_over_{beside}"] = {k: round(p[k] / d[k], 3) for k in p if k.endswith("_ms") and k in d}
     print(json.dumps(out), flush=True)
     return 0
 
@@ -471,10 +506,11 @@ def main() -> int:
     ap.add_argument("--workload", choices=sorted(WORKLOADS), help="instead of the default run: an engine workload of a "
                     "larger configuration (requests through the scheduler); --requests and --layers shrink it")
     ap.add_argument("--requests", type=int, default=0)
-    ap.add_argument("--design", choices=["pinorax", "rufedra"], help="instead of the default run: prefill and decode of another "
-                    "design of the framework beside the dense decoder at equal size (--size, --layers, --context)")
+    ap.add_argument("--design", choices=["pinorax", "rufedra", "dafalix"], help="instead of the default run: prefill and "
+                    "decode of another design of the framework beside the dense decoder (Dafalix: beside Rufedra) at "
+                    "equal size (--size, --layers, --context)")
     ap.add_argument("--size", choices=sorted(DESIGN_SIZES), default="s", help="of --design: s or l (see DESIGN_SIZES, "
-                    "RUFEDRA_SIZES)")
+                    "RUFEDRA_SIZES, DAFALIX_SIZES)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported by this single-GPU engine", flush=True)

@@ -142,6 +142,7 @@ struct GroupsParams {
   float limit, alpha;
   float up_offset;  // what the clamped up is raised by: 1 in the clamped form, 0 in the plain one
   int vec_store;
+  int c_f32;  // C holds 32-bit floats (the sums as they are) instead of bf16; strides count its elements
 };
 
 // A wave takes MT tiles of 16 tokens against NT tiles of 16 rows of W: every value it reads feeds MT or NT
@@ -245,6 +246,21 @@ __global__ void __launch_bounds__(256) gemm_groups_mfma_kernel(const GroupsParam
     if (am >= P.M) continue;
     uint16_t* cr = P.c + (size_t)group * P.c_group_stride + (size_t)am * P.ldc;
     const uint16_t* gr = P.gate ? P.gate + (size_t)group * P.c_group_stride + (size_t)am * P.ldg : nullptr;
+    if (P.c_f32) {  // no epilogue: the 32-bit sums go out unrounded
+      float* cf = (float*)P.c + (size_t)group * P.c_group_stride + (size_t)am * P.ldc;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        const int n = n0 + t * 16 + kb * 4;
+        if (P.vec_store && n + 3 < P.N) {
+          *(float4*)(cf + n) = make_float4(acc[mt][t][0], acc[mt][t][1], acc[mt][t][2], acc[mt][t][3]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (n + i < P.N) cf[n + i] = acc[mt][t][i];
+        }
+      }
+      continue;
+    }
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       const int n = n0 + t * 16 + kb * 4;
@@ -420,14 +436,16 @@ __global__ void __launch_bounds__(256) gemm_experts_lds_kernel(const GroupsParam
   }
 }
 
-// bf16 everywhere.  N: columns of C; with `glu` w holds 2 N rows a group.  groups > 0: the heads' form; 0: the
+// bf16 everywhere (c_f32: the results are the 32-bit sums).  N: columns of C; with `glu` w holds 2 N rows a group.  groups > 0: the heads' form; 0: the
 // experts' form with tiles of 16 * token_tiles rows.  token_tiles: 1 (few rows) or 4 (many).  K, the leading dimensions of a and w and the group strides of a and w must
 // be multiples of 8 and a, w lie on 16-byte boundaries (a lane reads 16 bytes at a time).
 extern "C" int rv_gemm_groups_mfma(hipStream_t stream, const void* a, const void* w, void* c, const int* row_index,
                                    const int* tile_group, int groups, int M, int N, int K, long long lda,
                                    long long ldw, long long ldc, long long a_group_stride, long long w_group_stride,
                                    long long c_group_stride, const void* gate, long long ldg, int glu, float limit,
-                                   float alpha, int token_tiles) {
+                                   float alpha, int token_tiles, int c_f32) {
+  RV_CHECK(!c_f32 || (groups > 0 && gate == nullptr && !glu),
+           "gemm_groups_mfma: 32-bit results come from the heads' form, without a gate or an activation");
   RV_CHECK(M >= 0 && N > 0 && K > 0 && groups >= 0, "gemm_groups_mfma: bad sizes M=%d N=%d K=%d groups=%d", M, N, K, groups);
   RV_CHECK((groups > 0) == (tile_group == nullptr), "gemm_groups_mfma: either a number of groups or the groups of the row tiles");
   RV_CHECK(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && a_group_stride % 8 == 0 && w_group_stride % 8 == 0 &&
@@ -451,7 +469,8 @@ extern "C" int rv_gemm_groups_mfma(hipStream_t stream, const void* a, const void
   P.a_group_stride = a_group_stride, P.w_group_stride = w_group_stride, P.c_group_stride = c_group_stride;
   P.limit = limit, P.alpha = alpha, P.up_offset = 1.0f;
   if (glu == 2) P.limit = __builtin_inff(), P.alpha = 1.0f, P.up_offset = 0.0f;  // silu(gate) * up, nothing clamped
-  P.vec_store = (ldc % 4 == 0 && c_group_stride % 4 == 0 && ((uintptr_t)c & 7) == 0) ? 1 : 0;
+  P.c_f32 = c_f32;
+  P.vec_store = (ldc % 4 == 0 && c_group_stride % 4 == 0 && ((uintptr_t)c & (c_f32 ? 15 : 7)) == 0) ? 1 : 0;
   if (groups == 0 && token_tiles == 4 && gate == nullptr) {  // the experts' products of many rows: tiles through LDS
     dim3 grid(rv_div_up(N, glu ? GL_BW / 2 : GL_BW), rv_div_up(M, GL_BM)), block(256);
     RV_CHECK(grid.y < 65536, "gemm_groups_mfma: too many row tiles for one launch");

@@ -327,7 +327,7 @@ def gemm_heads(a: torch.Tensor, a_col0: int, w: torch.Tensor, out: Optional[torc
         _check(library().rv_gemm_groups_mfma(
             _stream(), aptr, _ptr(w), _ptr(out), None, None, _c_int(heads), _c_int(m), _c_int(n), _c_int(k),
             _c_ll(a.stride(0)), _c_ll(k), _c_ll(out.stride(0)), _c_ll(k), _c_ll(n * k), _c_ll(n), gptr, _c_ll(ldg),
-            _c_int(0), _c_float(0.0), _c_float(0.0), _c_int(1 if m <= MFMA_GROUPS_FEW_ROWS else 4)))
+            _c_int(0), _c_float(0.0), _c_float(0.0), _c_int(1 if m <= MFMA_GROUPS_FEW_ROWS else 4), _c_int(0)))
         return out
     _check(library().rv_gemm_groups_plain(
         _stream(), aptr, _dt(a), _ptr(w), _dt(w), _ptr(out), _dt(out), None, None,
@@ -419,7 +419,7 @@ def gemm_experts(a: torch.Tensor, w: torch.Tensor, tile_group: torch.Tensor, row
         _check(library().rv_gemm_groups_mfma(
             _stream(), _ptr(a), _ptr(w), _ptr(out), _ptr(row_index), _ptr(tile_group), _c_int(0), _c_int(m), _c_int(n),
             _c_int(k), _c_ll(a.stride(0)), _c_ll(k), _c_ll(n), _c_ll(0), _c_ll(w.shape[1] * k), _c_ll(0), None, _c_ll(0),
-            _c_int(kind), _c_float(limit), _c_float(alpha), _c_int(tile // 16)))
+            _c_int(kind), _c_float(limit), _c_float(alpha), _c_int(tile // 16), _c_int(0)))
         return out
     _check(library().rv_gemm_groups_plain(
         _stream(), _ptr(a), _dt(a), _ptr(w), _dt(w), _ptr(out), _dt(out), _ptr(row_index), _ptr(tile_group), _c_int(0),
@@ -1845,6 +1845,12 @@ def gemm_blocks_f32(a: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     m = a.shape[0]
     _need(blocks * k == a.shape[1], "gemm_blocks_f32: the blocks' inputs fill the rows")
     out = torch.empty((m, blocks * n), dtype=torch.float32, device=a.device)
+    if a.dtype == torch.bfloat16 and _mfma_groups_take(a.data_ptr(), a.stride(0), w, k):  # on the matrix cores
+        _check(library().rv_gemm_groups_mfma(
+            _stream(), _ptr(a), _ptr(w), _ptr(out), None, None, _c_int(blocks), _c_int(m), _c_int(n), _c_int(k),
+            _c_ll(a.stride(0)), _c_ll(k), _c_ll(out.stride(0)), _c_ll(k), _c_ll(n * k), _c_ll(n), None, _c_ll(0),
+            _c_int(0), _c_float(0.0), _c_float(0.0), _c_int(1 if m <= MFMA_GROUPS_FEW_ROWS else 4), _c_int(1)))
+        return out
     _check(library().rv_gemm_groups_plain(
         _stream(), _ptr(a), _dt(a), _ptr(w), _dt(w), _ptr(out), _dt(out), None, None, _c_int(blocks), _c_int(m),
         _c_int(n), _c_int(k), _c_ll(a.stride(0)), _c_ll(k), _c_ll(out.stride(0)), _c_ll(k), _c_ll(n * k), _c_ll(n),
