@@ -614,44 +614,53 @@ extern "C" int rv_selective_scan(hipStream_t stream, const void* x, long long ld
 // ---------------------------------------------------------------------------
 // out[t][h][:] = o[t][h][:] / sqrt(mean(o[t][h][:]^2) + eps) * w[:] * act(gate[t][h][:]); a wave a (token, head).
 // o: float [tokens, heads dv]; gate: T, rows ld_gate apart; w: float [dv], shared by the heads, or (w_per_head)
-// [heads dv], every head its own; act 0: sigmoid, 1: silu; out: T.
+// [heads dv], every head its own; act 0: sigmoid, 1: silu; out: T.  With `dots` every head's o is first divided by
+// max(|dots[t][h]|, floors[(t heads + h) floor_stride]) + 1e-6: the divisor of a matrix memory's read-out.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ void __launch_bounds__(256)
 head_norm_gate_kernel(const float* __restrict__ o, const T* __restrict__ gate, long long ld_gate,
                       const float* __restrict__ w, T* __restrict__ out, int heads, int dv, float eps, long long units,
-                      int w_per_head, int act) {
+                      int w_per_head, int act, const float* __restrict__ dots, const float* __restrict__ floors,
+                      int floor_stride) {
   const int lane = threadIdx.x & (RV_WAVE - 1);
   const long long unit = (long long)blockIdx.x * (blockDim.x / RV_WAVE) + threadIdx.x / RV_WAVE;
   if (unit >= units) return;
   const long long t = unit / heads;
   const int h = (int)(unit - t * heads);
   const float* row = o + unit * dv;
+  const float den = dots ? fmaxf(fabsf(dots[unit]), floors[unit * floor_stride]) + 1e-6f : 1.0f;
   float ss = 0.f;
-  for (int d = lane; d < dv; d += RV_WAVE) ss = fmaf(row[d], row[d], ss);
+  for (int d = lane; d < dv; d += RV_WAVE) {
+    const float x = dots ? row[d] / den : row[d];
+    ss = fmaf(x, x, ss);
+  }
   ss = rv_wave_sum(ss);
   const float inv = 1.0f / sqrtf(ss / (float)dv + eps);
   for (int d = lane; d < dv; d += RV_WAVE) {
     const float gv = rv_to_float(gate[t * ld_gate + (long long)h * dv + d]);
     const float wv = w[w_per_head ? (long long)h * dv + d : d];
-    out[unit * dv + d] = rv_from_float<T>(row[d] * inv * wv * (act == 0 ? rec_sigmoid(gv) : rec_silu(gv)));
+    const float x = dots ? row[d] / den : row[d];
+    out[unit * dv + d] = rv_from_float<T>(x * inv * wv * (act == 0 ? rec_sigmoid(gv) : rec_silu(gv)));
   }
 }
 
 extern "C" int rv_head_norm_gate(hipStream_t stream, const float* o, const void* gate, long long ld_gate,
                                  const float* w, void* out, int dtype, int num_tokens, int heads, int dv, float eps,
-                                 int w_per_head, int act) {
+                                 int w_per_head, int act, const float* dots, const float* floors, int floor_stride) {
   RV_CHECK(o && gate && w && out && heads > 0 && dv > 0 && num_tokens >= 0 && (act == 0 || act == 1),
            "head_norm_gate: bad arguments");
+  RV_CHECK((dots == nullptr) == (floors == nullptr) && (dots == nullptr || floor_stride >= 1),
+           "head_norm_gate: a divisor takes the dots and their floors");
   if (num_tokens == 0) return 0;
   const long long units = (long long)num_tokens * heads;
   dim3 grid(rv_div_up(units, 4)), block(256);
   if (dtype == RV_F32)
     head_norm_gate_kernel<float><<<grid, block, 0, stream>>>(o, (const float*)gate, ld_gate, w, (float*)out, heads, dv,
-                                                             eps, units, w_per_head, act);
+                                                             eps, units, w_per_head, act, dots, floors, floor_stride);
   else if (dtype == RV_BF16)
     head_norm_gate_kernel<bf16_t><<<grid, block, 0, stream>>>(o, (const bf16_t*)gate, ld_gate, w, (bf16_t*)out, heads,
-                                                              dv, eps, units, w_per_head, act);
+                                                              dv, eps, units, w_per_head, act, dots, floors, floor_stride);
   else
     return rv_fail("head_norm_gate: unsupported dtype %d", dtype);
   RV_LAUNCH_CHECK("head_norm_gate");

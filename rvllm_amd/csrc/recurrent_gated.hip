@@ -4,10 +4,10 @@
 //   keeps the exponentials in range (m starts at 0):
 //       m' = max(f + m, i);  keep = e^(f + m - m'),  take = e^(i - m')
 //       S' = keep S + take k v^T;   n' = keep n + take k;   o = S'^T q / (max(|n' . q|, e^(-m')) + 1e-6)
-//     memory_gates   walks n and m (a vector and a number a head) and leaves keep, take and the divisor of every
-//                    token; the log gates come from capped inputs: i = cap tanh((a + b_i) / cap),
-//                    f = logsigmoid(cap tanh((a' + b_f) / cap))
-//     memory_matrix  walks S with these and reads it out
+//     memory_gates   walks m (a number a head) and leaves keep, take and e^(-m') of every token; the log gates
+//                    come from capped inputs: i = cap tanh((a + b_i) / cap), f = logsigmoid(cap tanh((a' + b_f) / cap))
+//     memory_matrix  walks S with these and reads it out; n is walked as one more column of S (a value of 1), whose
+//                    read-out is n' . q; the division is left to the kernel that norms the heads
 //
 //   gated linear recurrent unit (the real-gated LRU of Griffin), a channel at a time:
 //       r = sigmoid(g_r + b_r),  i = sigmoid(g_i + b_i),  log a = -8 r softplus(lam),  a = e^(log a)
@@ -40,118 +40,67 @@ __device__ __forceinline__ float rg_group_sum(float v) {
 }
 
 // ---------------------------------------------------------------------------
-// memory_gates.  A wave a (head, request); lane l holds the elements e * 64 + l of n.  The tokens' keys and queries
-// come CHUNK at a time into registers, a chunk ahead of the one worked on; a token's log gates are worked out by
-// the lane of its place in the chunk and handed round.
-//   rows  T [tokens, ld]: q of head h at q_col + h dk, k at k_col + h dk, the gates' inputs at i_col + h, f_col + h
-//   n [heads, dk] at n_off and m [heads] at m_off of the request's slot
-//   gates float [tokens, heads, 3]: keep, take, the divisor
+// memory_gates.  The running maximum is one number a head, walked token by token; everything else about a token's
+// gates is worked out side by side.  A wave a (head, request), 64 tokens at a time: lane l works out the log gates
+// of token l of the chunk, the maximum's walk (an add and a max a token) is done by all lanes alike with the
+// tokens' log gates handed round, and lane l then takes the exponentials of its token.
+//   rows   T [tokens, ld]: the gates' inputs of head h at i_col + h and f_col + h
+//   m [heads] at m_off of the request's slot
+//   gates  float [tokens, heads, 3]: keep = e^(f + m - m'), take = e^(i - m'), floor = e^(-m')
 // ---------------------------------------------------------------------------
-template <typename T, int PER, int CHUNK>
+template <typename T>
 __global__ void __launch_bounds__(RV_WAVE)
-memory_gates_kernel(const T* __restrict__ rows, long long ld, int q_col, int k_col, int i_col, int f_col,
-                    const float* __restrict__ i_bias, const float* __restrict__ f_bias, float cap, float q_scale,
-                    float* __restrict__ state, long long slot_stride, long long n_off, long long m_off,
-                    const int* __restrict__ q_start, const int* __restrict__ state_slot, float* __restrict__ gates,
-                    int heads, int dk) {
+memory_gates_kernel(const T* __restrict__ rows, long long ld, int i_col, int f_col, const float* __restrict__ i_bias,
+                    const float* __restrict__ f_bias, float cap, float* __restrict__ state, long long slot_stride,
+                    long long m_off, const int* __restrict__ q_start, const int* __restrict__ state_slot,
+                    float* __restrict__ gates, int heads) {
   const int lane = threadIdx.x;
   const int h = blockIdx.x;
   const int req = blockIdx.y;
-  float* slot = state + (long long)state_slot[req] * slot_stride;
-  float* n_mem = slot + n_off + (long long)h * dk;
-  float n[PER];
-#pragma unroll
-  for (int e = 0; e < PER; ++e) n[e] = e * RV_WAVE + lane < dk ? n_mem[e * RV_WAVE + lane] : 0.f;
-  float m = slot[m_off + h];
+  float* m_mem = state + (long long)state_slot[req] * slot_stride + m_off + h;
+  float m = *m_mem;
   const float bi = i_bias[h], bf = f_bias[h];
   const int t0 = q_start[req], t1 = q_start[req + 1];
-  float nk[CHUNK][PER], nq[CHUNK][PER], ngi = 0.f, ngf = 0.f;  // the chunk ahead
-  auto fetch = [&](int tb) {
-#pragma unroll
-    for (int c = 0; c < CHUNK; ++c) {
-#pragma unroll
-      for (int e = 0; e < PER; ++e) {
-        const int d = e * RV_WAVE + lane;
-        const bool ok = tb + c < t1 && d < dk;
-        const T* row = rows + (long long)(ok ? tb + c : t0) * ld + (long long)h * dk + (ok ? d : 0);
-        nk[c][e] = ok ? rv_to_float(row[k_col]) : 0.f;
-        nq[c][e] = ok ? rv_to_float(row[q_col]) * q_scale : 0.f;
-      }
-    }
-    const bool ok = lane < CHUNK && tb + lane < t1;
-    const T* row = rows + (long long)(ok ? tb + lane : t0) * ld + h;
-    ngi = rv_to_float(row[i_col]);
-    ngf = rv_to_float(row[f_col]);
-  };
-  if (t0 < t1) fetch(t0);
-  for (int tb = t0; tb < t1; tb += CHUNK) {
-    float k[CHUNK][PER], q[CHUNK][PER];
-#pragma unroll
-    for (int c = 0; c < CHUNK; ++c)
-#pragma unroll
-      for (int e = 0; e < PER; ++e) k[c][e] = nk[c][e], q[c][e] = nq[c][e];
-    const float log_in = cap * tanhf((ngi + bi) / cap);
-    const float capped = cap * tanhf((ngf + bf) / cap);
+  for (int tb = t0; tb < t1; tb += RV_WAVE) {
+    const int count = min(RV_WAVE, t1 - tb);
+    const bool mine = lane < count;
+    const T* row = rows + (long long)(mine ? tb + lane : t0) * ld + h;
+    const float log_in = cap * tanhf((rv_to_float(row[i_col]) + bi) / cap);
+    const float capped = cap * tanhf((rv_to_float(row[f_col]) + bf) / cap);
     const float log_forget = -rg_softplus(-capped);
-    if (tb + CHUNK < t1) fetch(tb + CHUNK);
-    const int count = min(CHUNK, t1 - tb);
-#pragma unroll
-    for (int c = 0; c < CHUNK; ++c) {
-      if (c < count) {
-        const float li = __shfl(log_in, c, RV_WAVE), lf = __shfl(log_forget, c, RV_WAVE);
-        const float m_new = fmaxf(lf + m, li);
-        const float keep = expf(lf + m - m_new), take = expf(li - m_new);
-        float dot = 0.f;
-#pragma unroll
-        for (int e = 0; e < PER; ++e) {
-          n[e] = fmaf(take, k[c][e], keep * n[e]);
-          dot = fmaf(n[e], q[c][e], dot);
-        }
-        dot = rv_wave_sum(dot);
-        m = m_new;
-        if (lane == 0) {
-          float* g = gates + ((long long)(tb + c) * heads + h) * 3;
-          g[0] = keep, g[1] = take, g[2] = fmaxf(fabsf(dot), expf(-m_new)) + 1e-6f;
-        }
-      }
+    float m_before = 0.f, m_after = 0.f;
+    for (int c = 0; c < count; ++c) {
+      const float li = __shfl(log_in, c, RV_WAVE), lf = __shfl(log_forget, c, RV_WAVE);
+      const float m_new = fmaxf(lf + m, li);
+      if (lane == c) m_before = m, m_after = m_new;
+      m = m_new;
+    }
+    if (mine) {
+      float* g = gates + ((long long)(tb + lane) * heads + h) * 3;
+      g[0] = expf(log_forget + m_before - m_after);
+      g[1] = expf(log_in - m_after);
+      g[2] = expf(-m_after);
     }
   }
-#pragma unroll
-  for (int e = 0; e < PER; ++e)
-    if (e * RV_WAVE + lane < dk) n_mem[e * RV_WAVE + lane] = n[e];
-  if (lane == 0) slot[m_off + h] = m;
+  if (lane == 0) *m_mem = m;
 }
 
-#define RG_GATES_PER_MAX 16
-
-extern "C" int rv_memory_gates(hipStream_t stream, const void* rows, int dtype, long long ld, int q_col, int k_col,
-                               int i_col, int f_col, const float* i_bias, const float* f_bias, float cap,
-                               float q_scale, float* state, long long slot_stride, long long n_off, long long m_off,
-                               const int* q_start, const int* state_slot, float* gates, int num_requests, int heads,
-                               int dk) {
+extern "C" int rv_memory_gates(hipStream_t stream, const void* rows, int dtype, long long ld, int i_col, int f_col,
+                               const float* i_bias, const float* f_bias, float cap, float* state,
+                               long long slot_stride, long long m_off, const int* q_start, const int* state_slot,
+                               float* gates, int num_requests, int heads) {
   RV_CHECK(rows && i_bias && f_bias && state && q_start && state_slot && gates, "memory_gates: null argument");
-  RV_CHECK(heads > 0 && dk > 0 && num_requests >= 0 && cap > 0.f, "memory_gates: bad sizes heads=%d dk=%d", heads, dk);
-  const int per = rv_div_up(dk, RV_WAVE);
-  RV_CHECK(per <= RG_GATES_PER_MAX, "memory_gates: a key size of %d is more than %d", dk, RG_GATES_PER_MAX * RV_WAVE);
+  RV_CHECK(heads > 0 && num_requests >= 0 && cap > 0.f, "memory_gates: bad sizes heads=%d", heads);
   if (num_requests == 0) return 0;
   dim3 grid(heads, num_requests), block(RV_WAVE);
-#define RV_MG(T, PER, CHUNK)                                                                                          \
-  memory_gates_kernel<T, PER, CHUNK><<<grid, block, 0, stream>>>((const T*)rows, ld, q_col, k_col, i_col, f_col, i_bias, \
-                                                                 f_bias, cap, q_scale, state, slot_stride, n_off, m_off, \
-                                                                 q_start, state_slot, gates, heads, dk)
-#define RV_MG_T(T)                              \
-  do {                                          \
-    if (per <= 1) RV_MG(T, 1, 16);              \
-    else if (per <= 2) RV_MG(T, 2, 16);         \
-    else if (per <= 4) RV_MG(T, 4, 8);          \
-    else if (per <= 8) RV_MG(T, 8, 4);          \
-    else RV_MG(T, 16, 2);                       \
-  } while (0)
-  if (dtype == RV_F32) RV_MG_T(float);
-  else if (dtype == RV_BF16) RV_MG_T(bf16_t);
-  else return rv_fail("memory_gates: unsupported dtype %d", dtype);
-#undef RV_MG_T
-#undef RV_MG
+  if (dtype == RV_F32)
+    memory_gates_kernel<float><<<grid, block, 0, stream>>>((const float*)rows, ld, i_col, f_col, i_bias, f_bias, cap,
+                                                           state, slot_stride, m_off, q_start, state_slot, gates, heads);
+  else if (dtype == RV_BF16)
+    memory_gates_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)rows, ld, i_col, f_col, i_bias, f_bias, cap,
+                                                            state, slot_stride, m_off, q_start, state_slot, gates, heads);
+  else
+    return rv_fail("memory_gates: unsupported dtype %d", dtype);
   RV_LAUNCH_CHECK("memory_gates");
   return 0;
 }
@@ -160,18 +109,21 @@ extern "C" int rv_memory_gates(hipStream_t stream, const void* rows, int dtype, 
 // memory_matrix.  A column j of a head's S (its dk numbers) never meets another column, so LANES neighbouring lanes
 // own one: lane `sub` of them holds rows sub * PER .. + PER.  A wave holds 64 / LANES columns of one head of one
 // request and walks the request's tokens of this step in order, CHUNK at a time through registers and LDS.
+// Column dv is n: its value is 1 for every token, it lives at n_off, and its read-out goes to `dots`.
 //   rows  T [tokens, ld]: q of head h at q_col + h dk, k at k_col + h dk, v at v_col + h dv
-//   gates float [tokens, heads, 3]: keep, take, the divisor (memory_gates)
+//   gates float [tokens, heads, 3]: keep, take, e^(-m') (memory_gates)
 //   S     float [heads, dv, dk] at s_off of the request's slot (a column's dk numbers side by side)
-//   out   float [tokens, heads dv]
+//   n     float [heads, dk] at n_off
+//   out   float [tokens, heads dv] = S'^T q, not yet divided;  dots float [tokens, heads] = n' . q
 // What a token's sums are does not depend on CHUNK: the same multiply-adds in the same order.
 // ---------------------------------------------------------------------------
 template <typename T, int PER, int LANES, int CHUNK>
 __global__ void __launch_bounds__(RV_WAVE)
 memory_matrix_kernel(const T* __restrict__ rows, long long ld, int q_col, int k_col, int v_col, float q_scale,
                      const float* __restrict__ gates, float* __restrict__ state, long long slot_stride,
-                     long long s_off, const int* __restrict__ q_start, const int* __restrict__ state_slot,
-                     float* __restrict__ out, int heads, int dk, int dv) {
+                     long long s_off, long long n_off, const int* __restrict__ q_start,
+                     const int* __restrict__ state_slot, float* __restrict__ out, float* __restrict__ dots, int heads,
+                     int dk, int dv) {
   constexpr int COLS = RV_WAVE / LANES;
   constexpr int DKP = PER * LANES;
   constexpr int NK = (CHUNK * DKP + RV_WAVE - 1) / RV_WAVE;
@@ -179,16 +131,18 @@ memory_matrix_kernel(const T* __restrict__ rows, long long ld, int q_col, int k_
   __shared__ __attribute__((aligned(16))) float sk[CHUNK][DKP];
   __shared__ __attribute__((aligned(16))) float sq[CHUNK][DKP];
   __shared__ float sv[CHUNK][COLS];
-  __shared__ float sg[CHUNK][3];
+  __shared__ float sg[CHUNK][2];
   const int lane = threadIdx.x;
   const int sub = lane % LANES;
   const int cl = lane / LANES;
   const int j = blockIdx.x * COLS + cl;
   const int h = blockIdx.y;
   const int req = blockIdx.z;
-  const bool col = j < dv;
-  const int jj = col ? j : dv - 1;  // a lane past the last column works on a copy and writes nothing
-  float* S_mem = state + (long long)state_slot[req] * slot_stride + s_off + ((long long)h * dv + jj) * dk + sub * PER;
+  const bool col = j <= dv;
+  const bool is_n = j == dv;
+  const int jj = j < dv ? j : dv - 1;  // a lane past the last column works on a copy and writes nothing
+  float* slot = state + (long long)state_slot[req] * slot_stride;
+  float* S_mem = (is_n ? slot + n_off + (long long)h * dk : slot + s_off + ((long long)h * dv + jj) * dk) + sub * PER;
   const bool vec = (dk % 4 == 0) && (((uintptr_t)S_mem & 15) == 0);
   float S[PER];
 #pragma unroll
@@ -219,10 +173,10 @@ memory_matrix_kernel(const T* __restrict__ rows, long long ld, int q_col, int k_
       const int tok = idx / COLS, c = idx % COLS;
       const int jc = blockIdx.x * COLS + c;
       const bool ok = tok < CHUNK && tb + tok < t1 && jc < dv;
-      rv[r] = ok ? rv_to_float(rows[(long long)(tb + tok) * ld + v_col + (long long)h * dv + jc]) : 0.f;
+      rv[r] = ok ? rv_to_float(rows[(long long)(tb + tok) * ld + v_col + (long long)h * dv + jc]) : (jc == dv ? 1.0f : 0.f);
     }
-    const int tok = lane / 3;
-    if (lane < CHUNK * 3 && tb + tok < t1) rg = gates[((long long)(tb + tok) * heads + h) * 3 + lane % 3];
+    const int tok = lane / 2;
+    if (lane < CHUNK * 2 && tb + tok < t1) rg = gates[((long long)(tb + tok) * heads + h) * 3 + lane % 2];
   };
   auto stage = [&]() {
 #pragma unroll
@@ -235,7 +189,7 @@ memory_matrix_kernel(const T* __restrict__ rows, long long ld, int q_col, int k_
       const int idx = r * RV_WAVE + lane;
       if (idx < CHUNK * COLS) (&sv[0][0])[idx] = rv[r];
     }
-    if (lane < CHUNK * 3) (&sg[0][0])[lane] = rg;
+    if (lane < CHUNK * 2) (&sg[0][0])[lane] = rg;
   };
   if (t0 < t1) fetch(t0);
   for (int tb = t0; tb < t1; tb += CHUNK) {
@@ -262,7 +216,10 @@ memory_matrix_kernel(const T* __restrict__ rows, long long ld, int q_col, int k_
         o = fmaf(S[e], qq[e], o);
       }
       o = rg_group_sum<LANES>(o);
-      if (col && sub == 0) out[(long long)(tb + t) * heads * dv + (long long)h * dv + j] = o / sg[t][2];
+      if (col && sub == 0) {
+        if (is_n) dots[(long long)(tb + t) * heads + h] = o;
+        else out[(long long)(tb + t) * heads * dv + (long long)h * dv + j] = o;
+      }
     }
   }
   if (col) {
@@ -294,21 +251,22 @@ static int rg_matrix_lanes(int dk) {
 // `longest`: the most tokens a request brings in this step (the size of the chunks is chosen by it).
 extern "C" int rv_memory_matrix(hipStream_t stream, const void* rows, int dtype, long long ld, int q_col, int k_col,
                                 int v_col, float q_scale, const float* gates, float* state, long long slot_stride,
-                                long long s_off, const int* q_start, const int* state_slot, float* out,
-                                int num_requests, int heads, int dk, int dv, int longest) {
-  RV_CHECK(rows && gates && state && q_start && state_slot && out, "memory_matrix: null argument");
+                                long long s_off, long long n_off, const int* q_start, const int* state_slot,
+                                float* out, float* dots, int num_requests, int heads, int dk, int dv, int longest) {
+  RV_CHECK(rows && gates && state && q_start && state_slot && out && dots, "memory_matrix: null argument");
   RV_CHECK(heads > 0 && dk > 0 && dv > 0 && num_requests >= 0, "memory_matrix: bad sizes heads=%d dk=%d dv=%d", heads,
            dk, dv);
   const int lanes = rg_matrix_lanes(dk);
   const int per = rv_div_up(dk, lanes);
   RV_CHECK(per <= RG_MATRIX_PER_MAX, "memory_matrix: a key size of %d is more than %d", dk, RG_MATRIX_PER_MAX * RV_WAVE);
   if (num_requests == 0) return 0;
-  dim3 grid(rv_div_up(dv, RV_WAVE / lanes), heads, num_requests), block(RV_WAVE);
+  dim3 grid(rv_div_up(dv + 1, RV_WAVE / lanes), heads, num_requests), block(RV_WAVE);  // the values' columns and n
   const bool few = longest <= 2;  // decoded tokens: small chunks, little LDS, more waves a CU
 #define RV_MM(T, PER, LANES, CHUNK)                                                                               \
   memory_matrix_kernel<T, PER, LANES, CHUNK><<<grid, block, 0, stream>>>((const T*)rows, ld, q_col, k_col, v_col, \
                                                                          q_scale, gates, state, slot_stride, s_off, \
-                                                                         q_start, state_slot, out, heads, dk, dv)
+                                                                         n_off, q_start, state_slot, out, dots, heads, \
+                                                                         dk, dv)
 #define RV_MM_L(T, PER, LANES, CHUNK)          \
   do {                                         \
     if (few) RV_MM(T, PER, LANES, 2);          \
@@ -337,8 +295,13 @@ extern "C" int rv_memory_matrix(hipStream_t stream, const void* rows, int dtype,
 }
 
 // ---------------------------------------------------------------------------
-// gated_linear_scan.  A lane a channel of a request; the tokens' operands come CHUNK at a time into registers, a
-// chunk ahead of the one worked on.  1 - a^2 is taken as -expm1(2 log a), which keeps its digits where a is near 1.
+// gated_linear_scan.  A lane a channel of a request.  1 - a^2 is taken as -expm1(2 log a), which keeps its digits
+// where a is near 1.  What a token brings to the walk (its decay a, its input x = sqrt(1 - a^2) i u and the other
+// branch's activation) does not wait for S, only S' = a S + x does:
+//   few tokens a request (decoding): one kernel, a token's terms worked out where it is walked;
+//   many (prompts): the terms of all tokens and channels side by side by one launch (gated_linear_terms), then the
+//   walk alone, CHUNK tokens' terms in registers a chunk ahead: three reads, a multiply-add and a product a token.
+// Both ways a token's terms come from the same function and its S from the same chain of multiply-adds.
 //   u      T [tokens, ld_u]      the convolved input
 //   gates  float [tokens, ld_g]  channel c = b * block + j: g_r at b * 2 block + j, g_i at b * 2 block + block + j
 //                                (what a product by blocks against each block's two matrices, one after the other,
@@ -347,7 +310,16 @@ extern "C" int rv_memory_matrix(hipStream_t stream, const void* rows, int dtype,
 //   S      float [channels] at s_off of the request's slot
 //   out    T [tokens, channels] = S' * gelu_tanh(y), the activation rounded to T first
 // ---------------------------------------------------------------------------
-template <typename T, int CHUNK>
+template <typename T>
+__device__ __forceinline__ void rg_unit_terms(float u, float g_r, float g_i, float y, float rate, float br, float bi,
+                                              float& a, float& x, float& gy) {
+  const float log_a = rate * rg_sigmoid(g_r + br);
+  a = expf(log_a);
+  x = sqrtf(-expm1f(2.0f * log_a)) * rg_sigmoid(g_i + bi) * u;
+  gy = rv_round_to<T>(rv_gated<float, 0>(y, 1.0f));
+}
+
+template <typename T>
 __global__ void __launch_bounds__(RV_WAVE)
 gated_linear_scan_kernel(const T* __restrict__ u, long long ld_u, const float* __restrict__ gates, long long ld_g,
                          int block_size, const float* __restrict__ r_bias, const float* __restrict__ i_bias,
@@ -357,69 +329,121 @@ gated_linear_scan_kernel(const T* __restrict__ u, long long ld_u, const float* _
                          int channels) {
   const int ch = blockIdx.x * RV_WAVE + threadIdx.x;
   const int req = blockIdx.y;
-  const bool live = ch < channels;
-  const int c = live ? ch : channels - 1;
-  const int b = c / block_size, jn = c - b * block_size;
+  if (ch >= channels) return;
+  const int b = ch / block_size, jn = ch - b * block_size;
   const long long g_r = (long long)b * 2 * block_size + jn, g_i = g_r + block_size;
-  float* S_mem = state + (long long)state_slot[req] * slot_stride + s_off + c;
+  float* S_mem = state + (long long)state_slot[req] * slot_stride + s_off + ch;
   float S = *S_mem;
-  const float rate = -8.0f * rg_softplus(lam[c]);
-  const float br = r_bias[c], bi = i_bias[c];
+  const float rate = -8.0f * rg_softplus(lam[ch]);
+  const float br = r_bias[ch], bi = i_bias[ch];
   const int t0 = q_start[req], t1 = q_start[req + 1];
-  float nu[CHUNK], nr[CHUNK], ni[CHUNK], ny[CHUNK];
+  for (long long t = t0; t < t1; ++t) {
+    float a, x, gy;
+    rg_unit_terms<T>(rv_to_float(u[t * ld_u + ch]), gates[t * ld_g + g_r], gates[t * ld_g + g_i],
+                     rv_to_float(y[t * ld_y + ch]), rate, br, bi, a, x, gy);
+    S = fmaf(a, S, x);
+    out[t * channels + ch] = rv_from_float<T>(S * gy);
+  }
+  *S_mem = S;
+}
+
+// terms: float [2, tokens, channels] (a, then x); act: T [tokens, channels]
+template <typename T>
+__global__ void __launch_bounds__(256)
+gated_linear_terms_kernel(const T* __restrict__ u, long long ld_u, const float* __restrict__ gates, long long ld_g,
+                          int block_size, const float* __restrict__ r_bias, const float* __restrict__ i_bias,
+                          const float* __restrict__ lam, const T* __restrict__ y, long long ld_y,
+                          float* __restrict__ terms, T* __restrict__ act, int num_tokens, int channels) {
+  const int ch = blockIdx.x * 256 + threadIdx.x;
+  const long long t = blockIdx.y;
+  if (ch >= channels) return;
+  const int b = ch / block_size, jn = ch - b * block_size;
+  const long long g_r = (long long)b * 2 * block_size + jn, g_i = g_r + block_size;
+  const float rate = -8.0f * rg_softplus(lam[ch]);
+  float a, x, gy;
+  rg_unit_terms<T>(rv_to_float(u[t * ld_u + ch]), gates[t * ld_g + g_r], gates[t * ld_g + g_i],
+                   rv_to_float(y[t * ld_y + ch]), rate, r_bias[ch], i_bias[ch], a, x, gy);
+  terms[t * channels + ch] = a;
+  terms[((long long)num_tokens + t) * channels + ch] = x;
+  act[t * channels + ch] = rv_from_float<T>(gy);
+}
+
+template <typename T, int CHUNK>
+__global__ void __launch_bounds__(RV_WAVE)
+gated_linear_walk_kernel(const float* __restrict__ terms, const T* __restrict__ act, float* __restrict__ state,
+                         long long slot_stride, long long s_off, const int* __restrict__ q_start,
+                         const int* __restrict__ state_slot, T* __restrict__ out, int num_tokens, int channels) {
+  const int ch = blockIdx.x * RV_WAVE + threadIdx.x;
+  const int req = blockIdx.y;
+  if (ch >= channels) return;
+  float* S_mem = state + (long long)state_slot[req] * slot_stride + s_off + ch;
+  float S = *S_mem;
+  const float* ta = terms + ch;
+  const float* tx = terms + (long long)num_tokens * channels + ch;
+  const int t0 = q_start[req], t1 = q_start[req + 1];
+  float na[CHUNK], nx[CHUNK], ng[CHUNK];
   auto fetch = [&](int tb) {
 #pragma unroll
     for (int k = 0; k < CHUNK; ++k) {
       const long long t = tb + k < t1 ? tb + k : t0;
-      nu[k] = rv_to_float(u[t * ld_u + c]);
-      nr[k] = gates[t * ld_g + g_r];
-      ni[k] = gates[t * ld_g + g_i];
-      ny[k] = rv_to_float(y[t * ld_y + c]);
+      na[k] = ta[t * channels];
+      nx[k] = tx[t * channels];
+      ng[k] = rv_to_float(act[t * channels + ch]);
     }
   };
   if (t0 < t1) fetch(t0);
   for (int tb = t0; tb < t1; tb += CHUNK) {
     float a[CHUNK], x[CHUNK], gy[CHUNK];
 #pragma unroll
-    for (int k = 0; k < CHUNK; ++k) {  // nothing here waits for S: the tokens' decays and inputs side by side
-      const float log_a = rate * rg_sigmoid(nr[k] + br);
-      a[k] = expf(log_a);
-      x[k] = sqrtf(-expm1f(2.0f * log_a)) * rg_sigmoid(ni[k] + bi) * nu[k];
-      gy[k] = rv_round_to<T>(rv_gated<float, 0>(ny[k], 1.0f));
-    }
+    for (int k = 0; k < CHUNK; ++k) a[k] = na[k], x[k] = nx[k], gy[k] = ng[k];
     if (tb + CHUNK < t1) fetch(tb + CHUNK);
     const int count = min(CHUNK, t1 - tb);
 #pragma unroll
     for (int k = 0; k < CHUNK; ++k) {
       if (k < count) {
         S = fmaf(a[k], S, x[k]);
-        if (live) out[(long long)(tb + k) * channels + ch] = rv_from_float<T>(S * gy[k]);
+        out[(long long)(tb + k) * channels + ch] = rv_from_float<T>(S * gy[k]);
       }
     }
   }
-  if (live) *S_mem = S;
+  *S_mem = S;
 }
 
+// `terms` (float [2, tokens, channels]) and `act` (of `dtype`, [tokens, channels]) are scratch for the two-launch
+// form; null: the one-launch form.
 extern "C" int rv_gated_linear_scan(hipStream_t stream, const void* u, long long ld_u, const float* gates,
                                     long long ld_g, int block_size, const float* r_bias, const float* i_bias,
                                     const float* lam, const void* y, long long ld_y, float* state,
                                     long long slot_stride, long long s_off, const int* q_start, const int* state_slot,
-                                    void* out, int dtype, int num_requests, int channels, int longest) {
+                                    void* out, int dtype, int num_requests, int num_tokens, int channels, float* terms,
+                                    void* act) {
   RV_CHECK(u && gates && r_bias && i_bias && lam && y && state && q_start && state_slot && out,
            "gated_linear_scan: null argument");
-  RV_CHECK(channels > 0 && block_size > 0 && channels % block_size == 0 && num_requests >= 0 && ld_u >= channels &&
-               ld_y >= channels && ld_g >= 2LL * channels,
+  RV_CHECK(channels > 0 && block_size > 0 && channels % block_size == 0 && num_requests >= 0 && num_tokens >= 0 &&
+               ld_u >= channels && ld_y >= channels && ld_g >= 2LL * channels,
            "gated_linear_scan: bad sizes channels=%d block=%d", channels, block_size);
-  if (num_requests == 0) return 0;
+  RV_CHECK((terms == nullptr) == (act == nullptr), "gated_linear_scan: the scratch is both or neither");
+  RV_CHECK(dtype == RV_F32 || dtype == RV_BF16, "gated_linear_scan: unsupported dtype %d", dtype);
+  if (num_requests == 0 || num_tokens == 0) return 0;
   dim3 grid(rv_div_up(channels, RV_WAVE), num_requests), block(RV_WAVE);
-  const bool few = longest <= 2;
-#define RV_GS(T, CHUNK)                                                                                            \
-  gated_linear_scan_kernel<T, CHUNK><<<grid, block, 0, stream>>>((const T*)u, ld_u, gates, ld_g, block_size, r_bias, \
-                                                                 i_bias, lam, (const T*)y, ld_y, state, slot_stride, \
-                                                                 s_off, q_start, state_slot, (T*)out, channels)
-  if (dtype == RV_F32) { if (few) RV_GS(float, 1); else RV_GS(float, 8); }
-  else if (dtype == RV_BF16) { if (few) RV_GS(bf16_t, 1); else RV_GS(bf16_t, 8); }
-  else return rv_fail("gated_linear_scan: unsupported dtype %d", dtype);
+#define RV_GS(T)                                                                                                     \
+  do {                                                                                                               \
+    if (terms == nullptr) {                                                                                          \
+      gated_linear_scan_kernel<T><<<grid, block, 0, stream>>>((const T*)u, ld_u, gates, ld_g, block_size, r_bias,    \
+                                                              i_bias, lam, (const T*)y, ld_y, state, slot_stride,    \
+                                                              s_off, q_start, state_slot, (T*)out, channels);        \
+    } else {                                                                                                         \
+      RV_CHECK(num_tokens < 65536, "gated_linear_scan: %d tokens are too many for one launch", num_tokens);          \
+      gated_linear_terms_kernel<T><<<dim3(rv_div_up(channels, 256), num_tokens), dim3(256), 0, stream>>>(            \
+          (const T*)u, ld_u, gates, ld_g, block_size, r_bias, i_bias, lam, (const T*)y, ld_y, terms, (T*)act,        \
+          num_tokens, channels);                                                                                     \
+      gated_linear_walk_kernel<T, 16><<<grid, block, 0, stream>>>(terms, (const T*)act, state, slot_stride, s_off,   \
+                                                                  q_start, state_slot, (T*)out, num_tokens,          \
+                                                                  channels);                                         \
+    }                                                                                                                \
+  } while (0)
+  if (dtype == RV_F32) RV_GS(float);
+  else RV_GS(bf16_t);
 #undef RV_GS
   RV_LAUNCH_CHECK("gated_linear_scan");
   return 0;

@@ -144,11 +144,14 @@ struct StreamsParams {
   float eps;
 };
 
-template <typename T, int E>
+// ST: the number of streams where it is one of the usual few (their sums are then written out in registers), 0: any
+// number up to SN_MAX_STREAMS.  A stream's sum over the old streams is added in their order either way.
+template <typename T, int E, int ST>
 __global__ void __launch_bounds__(SN_THREADS) streams_update_kernel(StreamsParams P) {
   __shared__ float scratch[16];
   __shared__ float s_mix[SN_MAX_STREAMS * SN_MAX_STREAMS], s_out[SN_MAX_STREAMS], s_in[SN_MAX_STREAMS];
-  const int S = P.S, width = P.width;
+  constexpr int SMAX = ST > 0 ? ST : SN_MAX_STREAMS;
+  const int S = ST > 0 ? ST : P.S, width = P.width;
   const size_t row0 = (size_t)blockIdx.x * width;
   if (threadIdx.x < S * S) s_mix[threadIdx.x] = P.branch ? P.mix[threadIdx.x] : 0.f;
   if (threadIdx.x < S) {
@@ -160,32 +163,32 @@ __global__ void __launch_bounds__(SN_THREADS) streams_update_kernel(StreamsParam
   float u[N];
   // one element of the row: its streams moved on and written, the next sublayer's input returned
   auto element = [&](int i) -> float {
-    float old[SN_MAX_STREAMS], fresh[SN_MAX_STREAMS];
+    float old[SMAX], fresh[SMAX];
 #pragma unroll
-    for (int s = 0; s < SN_MAX_STREAMS; ++s)
+    for (int s = 0; s < SMAX; ++s)
       if (s < S) old[s] = P.seed ? P.seed[row0 + i] : P.streams[(size_t)s * P.stream_stride + row0 + i];
     if (P.branch) {
       float y = sn_branch<T>(P.branch, P.slices, P.slice_stride, row0 + i);
       if (P.branch2) y = P.wa * y + P.wb * sn_branch<T>(P.branch2, P.slices2, P.slice_stride2, row0 + i);
       if (P.layer_scale) y *= P.layer_scale[i];
 #pragma unroll
-      for (int t = 0; t < SN_MAX_STREAMS; ++t) {
+      for (int t = 0; t < SMAX; ++t) {
         if (t < S) {
           float acc = 0.f;
 #pragma unroll
-          for (int s = 0; s < SN_MAX_STREAMS; ++s)
+          for (int s = 0; s < SMAX; ++s)
             if (s < S) acc = fmaf(s_mix[s * S + t], old[s], acc);
           fresh[t] = fmaf(s_out[t], y, acc);
         }
       }
     } else {
 #pragma unroll
-      for (int s = 0; s < SN_MAX_STREAMS; ++s)
+      for (int s = 0; s < SMAX; ++s)
         if (s < S) fresh[s] = old[s];
     }
     float in_sum = 0.f, all = 0.f;
 #pragma unroll
-    for (int s = 0; s < SN_MAX_STREAMS; ++s) {
+    for (int s = 0; s < SMAX; ++s) {
       if (s < S) {
         if (P.branch || P.seed) P.streams[(size_t)s * P.stream_stride + row0 + i] = fresh[s];
         in_sum = fmaf(s_in[s], fresh[s], in_sum);
@@ -261,18 +264,27 @@ extern "C" int rv_streams_update(hipStream_t stream, float* streams, long long s
   P.norm_w = norm_w, P.norm_b = norm_b, P.norm_f32 = norm_f32, P.next = next, P.total = total, P.S = num_streams;
   P.width = width, P.eps = eps;
   dim3 grid(rows), block(SN_THREADS);
-#define RV_SU_T(T)                                                                       \
-  do {                                                                                   \
-    const int e_ = rv_div_up(width, SN_THREADS);                                         \
-    if (e_ <= 1) streams_update_kernel<T, 1><<<grid, block, 0, stream>>>(P);             \
-    else if (e_ <= 4) streams_update_kernel<T, 4><<<grid, block, 0, stream>>>(P);        \
-    else if (e_ <= 16) streams_update_kernel<T, 16><<<grid, block, 0, stream>>>(P);      \
-    else streams_update_kernel<T, 0><<<grid, block, 0, stream>>>(P);                     \
+#define RV_SU_S(T, E)                                                                            \
+  do {                                                                                           \
+    if (num_streams == 1) streams_update_kernel<T, E, 1><<<grid, block, 0, stream>>>(P);         \
+    else if (num_streams == 2) streams_update_kernel<T, E, 2><<<grid, block, 0, stream>>>(P);    \
+    else if (num_streams == 4) streams_update_kernel<T, E, 4><<<grid, block, 0, stream>>>(P);    \
+    else streams_update_kernel<T, E, 0><<<grid, block, 0, stream>>>(P);                          \
+  } while (0)
+#define RV_SU_T(T)                                   \
+  do {                                               \
+    const int e_ = rv_div_up(width, SN_THREADS);     \
+    if (e_ <= 1) RV_SU_S(T, 1);                      \
+    else if (e_ <= 4) RV_SU_S(T, 4);                 \
+    else if (e_ <= 8) RV_SU_S(T, 8);                 \
+    else if (e_ <= 16) RV_SU_S(T, 16);               \
+    else RV_SU_S(T, 0);                              \
   } while (0)
   if (dtype == RV_F32) RV_SU_T(float);
   else if (dtype == RV_BF16) RV_SU_T(bf16_t);
   else return rv_fail("streams_update: unsupported dtype %d", dtype);
 #undef RV_SU_T
+#undef RV_SU_S
   RV_LAUNCH_CHECK("streams_update");
   return 0;
 }

@@ -1643,9 +1643,11 @@ def delta_rule(qkv: torch.Tensor, q_off: int, k_off: int, v_off: int, ab: torch.
 
 
 def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, gate_col0: int, weight: torch.Tensor, eps: float, heads: int,
-                   dv: int, out_dtype: torch.dtype, act: str = "silu") -> torch.Tensor:
+                   dv: int, out_dtype: torch.dtype, act: str = "silu", divisor=None) -> torch.Tensor:
     """out[t, h] = o[t, h] / rms(o[t, h]) * weight * act(gate[t, gate_col0 + h dv ...]) for every head; ``weight`` is
-    ``[dv]``, shared by the heads, or ``[heads * dv]``, every head its own; ``act`` is ``silu`` or ``sigmoid``."""
+    ``[dv]``, shared by the heads, or ``[heads * dv]``, every head its own; ``act`` is ``silu`` or ``sigmoid``.
+    ``divisor`` = (dots float32 ``[tokens, heads]``, gates float32 ``[tokens, heads, 3]``): every head's o is first
+    divided by max(|dot|, gates[..., 2]) + 1e-6 (what ``matrix_memory`` leaves undivided)."""
     _gpu(o, weight)
     n = o.shape[0]
     _need(o.dtype == torch.float32 and o.shape == (n, heads * dv), "head_norm_gate: float32 [tokens, heads * dv]")
@@ -1656,9 +1658,17 @@ def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, gate_col0: int, weight: 
     _need(gate.is_cuda and gate.dim() == 2 and gate.stride(1) == 1 and gate.dtype == out_dtype and gate.shape[0] == n
           and 0 <= gate_col0 and gate_col0 + heads * dv <= gate.shape[1], "head_norm_gate: the gate lies outside its rows")
     out = torch.empty((n, heads * dv), dtype=out_dtype, device=o.device)
+    dots = floors = None
+    if divisor is not None:
+        dots, gates = divisor
+        _gpu(dots, gates)
+        _need(dots.shape == (n, heads) and gates.shape == (n, heads, 3) and dots.dtype == gates.dtype == torch.float32
+              and dots.is_contiguous() and gates.is_contiguous(), "head_norm_gate: float32 dots [tokens, heads] and gates")
+        floors = gates.data_ptr() + 2 * gates.element_size()
     _check(library().rv_head_norm_gate(_stream(), _ptr(o), gate.data_ptr() + gate_col0 * gate.element_size(),
                                        _c_ll(gate.stride(0)), _ptr(weight), _ptr(out), _dt(out), _c_int(n), _c_int(heads),
-                                       _c_int(dv), _c_float(eps), _c_int(per_head), _c_int(GATE_ACTS[act])))
+                                       _c_int(dv), _c_float(eps), _c_int(per_head), _c_int(GATE_ACTS[act]), _ptr(dots),
+                                       floors, _c_int(3)))
     return out
 
 
@@ -1770,14 +1780,15 @@ def streams_update(streams: torch.Tensor, out_dtype: torch.dtype, *, seed: Optio
 # ---- a matrix memory with log gates; a gated linear recurrent unit -----------------------------------------------
 def matrix_memory(rows: torch.Tensor, q_col: int, k_col: int, v_col: int, i_col: int, f_col: int, i_bias: torch.Tensor,
                   f_bias: torch.Tensor, cap: float, q_scale: float, slots: torch.Tensor, s_off: int, n_off: int,
-                  m_off: int, step, heads: int, dk: int, dv: int) -> torch.Tensor:
+                  m_off: int, step, heads: int, dk: int, dv: int) -> tuple[torch.Tensor, tuple]:
     """The matrix memory over the step's tokens, request by request in order.  The rows hold, head after head,
     queries at ``q_col`` and keys at ``k_col`` (``dk`` a head), values at ``v_col`` (``dv`` a head) and the two
     gates' inputs at ``i_col + h`` and ``f_col + h``.  Log gates i = cap tanh((a_i + i_bias) / cap),
     f = logsigmoid(cap tanh((a_f + f_bias) / cap)); m' = max(f + m, i); S' = e^(f + m - m') S + e^(i - m') k v^T, n
     likewise with k alone; o = S'^T q / (max(|n' . q|, e^(-m')) + 1e-6), q times ``q_scale``.  In the request's
     32-bit slot S lies at ``s_off`` as ``[heads, dv, dk]``, n at ``n_off`` ``[heads, dk]``, m at ``m_off`` ``[heads]``.
-    Returns o as float32 ``[tokens, heads * dv]``."""
+    Returns (S'^T q as float32 ``[tokens, heads * dv]``, not yet divided; the divisor's parts (n' . q ``[tokens,
+    heads]``, gates ``[tokens, heads, 3]`` whose last entry is e^(-m'))): ``head_norm_gate(..., divisor=)`` divides."""
     _gpu(i_bias, f_bias)
     n = rows.shape[0]
     _need(rows.is_cuda and rows.dim() == 2 and rows.stride(1) == 1 and rows.dtype in _DT and n == step.num_tokens,
@@ -1792,19 +1803,22 @@ def matrix_memory(rows: torch.Tensor, q_col: int, k_col: int, v_col: int, i_col:
     _need(0 <= s_off and s_off + heads * dk * dv <= size and 0 <= n_off and n_off + heads * dk <= size
           and 0 <= m_off and m_off + heads <= size, "matrix_memory: the state lies outside the slot")
     gates = torch.empty((n, heads, 3), dtype=torch.float32, device=rows.device)
+    dots = torch.empty((n, heads), dtype=torch.float32, device=rows.device)
     out = torch.empty((n, heads * dv), dtype=torch.float32, device=rows.device)
     lib = library()
     _check(lib.rv_memory_gates(
-        _stream(), _ptr(rows), _dt(rows), _c_ll(rows.stride(0)), _c_int(q_col), _c_int(k_col), _c_int(i_col),
-        _c_int(f_col), _ptr(i_bias), _ptr(f_bias), _c_float(cap), _c_float(q_scale), _ptr(slots), _c_ll(stride),
-        _c_ll(n_off), _c_ll(m_off), _ptr(step.q_start), _ptr(step.state_slot), _ptr(gates), _c_int(step.num_requests),
-        _c_int(heads), _c_int(dk)))
+        _stream(), _ptr(rows), _dt(rows), _c_ll(rows.stride(0)), _c_int(i_col), _c_int(f_col), _ptr(i_bias),
+        _ptr(f_bias), _c_float(cap), _ptr(slots), _c_ll(stride), _c_ll(m_off), _ptr(step.q_start),
+        _ptr(step.state_slot), _ptr(gates), _c_int(step.num_requests), _c_int(heads)))
     _check(lib.rv_memory_matrix(
         _stream(), _ptr(rows), _dt(rows), _c_ll(rows.stride(0)), _c_int(q_col), _c_int(k_col), _c_int(v_col),
-        _c_float(q_scale), _ptr(gates), _ptr(slots), _c_ll(stride), _c_ll(s_off), _ptr(step.q_start),
-        _ptr(step.state_slot), _ptr(out), _c_int(step.num_requests), _c_int(heads), _c_int(dk), _c_int(dv),
+        _c_float(q_scale), _ptr(gates), _ptr(slots), _c_ll(stride), _c_ll(s_off), _c_ll(n_off), _ptr(step.q_start),
+        _ptr(step.state_slot), _ptr(out), _ptr(dots), _c_int(step.num_requests), _c_int(heads), _c_int(dk), _c_int(dv),
         _c_int(step.max_portion)))
-    return out
+    return out, (dots, gates)
+
+
+GATED_SCAN_FEW = 4  # tokens a request up to which the recurrent unit's walk works its terms out itself
 
 
 def gated_linear_scan(u: torch.Tensor, gates: torch.Tensor, block: int, r_bias: torch.Tensor, i_bias: torch.Tensor,
@@ -1828,11 +1842,15 @@ def gated_linear_scan(u: torch.Tensor, gates: torch.Tensor, block: int, r_bias: 
     stride = _state_args(slots, "gated_linear_scan")
     _need(0 <= s_off and s_off + channels <= slots.shape[1], "gated_linear_scan: the state lies outside the slot")
     out = torch.empty((n, channels), dtype=u.dtype, device=u.device)
+    terms = act = None
+    if step.max_portion > GATED_SCAN_FEW:  # prompts: every token's terms by one launch, then the walk alone
+        terms = torch.empty((2, n, channels), dtype=torch.float32, device=u.device)
+        act = torch.empty((n, channels), dtype=u.dtype, device=u.device)
     _check(library().rv_gated_linear_scan(
         _stream(), _ptr(u), _c_ll(u.stride(0)), _ptr(gates), _c_ll(gates.stride(0)), _c_int(block), _ptr(r_bias),
         _ptr(i_bias), _ptr(lam), y.data_ptr() + y_col0 * y.element_size(), _c_ll(y.stride(0)), _ptr(slots),
         _c_ll(stride), _c_ll(s_off), _ptr(step.q_start), _ptr(step.state_slot), _ptr(out), _dt(u),
-        _c_int(step.num_requests), _c_int(channels), _c_int(step.max_portion)))
+        _c_int(step.num_requests), _c_int(n), _c_int(channels), _ptr(terms), _ptr(act)))
     return out
 
 

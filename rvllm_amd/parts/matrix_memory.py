@@ -95,11 +95,11 @@ class MatrixMemory(Mixer):
         if not cache.writes:
             raise ValueError("a matrix-memory layer moves its state on with every token and cannot read another's")
         proj = linear(x, self.w_in)  # [n, q | k | v | g | i | f]
-        o = ops.matrix_memory(proj, 0, self.k_col, self.v_col, self.i_col, self.f_col, self.i_bias, self.f_bias,
+        o, divisor = ops.matrix_memory(proj, 0, self.k_col, self.v_col, self.i_col, self.f_col, self.i_bias, self.f_bias,
                               self.cap, self.dim ** -0.5, cache.slots, 0, self.n_off, self.m_off, step, self.heads,
                               self.dim, self.vdim)
         y = ops.head_norm_gate(o, proj, self.g_col, self.norm_w, self.eps, self.heads, self.vdim, x.dtype,
-                               act="sigmoid")
+                               act="sigmoid", divisor=divisor)
         return linear_unrounded(y, self.w_o)
 
 
