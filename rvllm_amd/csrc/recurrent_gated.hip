@@ -70,7 +70,9 @@ memory_gates_kernel(const T* __restrict__ rows, long long ld, int i_col, int f_c
     const float log_forget = -rg_softplus(-capped);
     float m_before = 0.f, m_after = 0.f;
     for (int c = 0; c < count; ++c) {
-      const float li = __shfl(log_in, c, RV_WAVE), lf = __shfl(log_forget, c, RV_WAVE);
+      // token c's log gates from lane c: c is the same in every lane, so a read of that lane's register
+      const float li = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, log_in), c));
+      const float lf = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, log_forget), c));
       const float m_new = fmaxf(lf + m, li);
       if (lane == c) m_before = m, m_after = m_new;
       m = m_new;
@@ -155,8 +157,14 @@ memory_matrix_kernel(const T* __restrict__ rows, long long ld, int q_col, int k_
       for (int u = 0; u < 4; ++u) S[e + u] = sub * PER + e + u < dk ? S_mem[e + u] : 0.f;
     }
   }
+  float* dst = is_n ? dots + h : out + (long long)h * dv + jj;  // where a token's read-out goes, rows dst_stride apart
+  const long long dst_stride = is_n ? heads : (long long)heads * dv;
   const int t0 = q_start[req], t1 = q_start[req + 1];
-  float rk[NK], rq[NK], rv[NV], rg = 0.f;
+  // A chunk's operands as they lie in memory, read without a condition from addresses that exist (a token past the
+  // request's end reads the first one's, a dimension past dk the first), so that no read waits for the one before;
+  // they become numbers, with zeros where nothing is, when they go into LDS.
+  T rk[NK], rq[NK], rv[NV];
+  float rg = 0.f;
   auto fetch = [&](int tb) {
 #pragma unroll
     for (int r = 0; r < NK; ++r) {
@@ -164,8 +172,8 @@ memory_matrix_kernel(const T* __restrict__ rows, long long ld, int q_col, int k_
       const int tok = idx / DKP, i = idx % DKP;
       const bool ok = tok < CHUNK && tb + tok < t1 && i < dk;
       const T* row = rows + (long long)(ok ? tb + tok : t0) * ld + (long long)h * dk + (ok ? i : 0);
-      rk[r] = ok ? rv_to_float(row[k_col]) : 0.f;
-      rq[r] = ok ? rv_to_float(row[q_col]) * q_scale : 0.f;
+      rk[r] = row[k_col];
+      rq[r] = row[q_col];
     }
 #pragma unroll
     for (int r = 0; r < NV; ++r) {
@@ -173,28 +181,37 @@ memory_matrix_kernel(const T* __restrict__ rows, long long ld, int q_col, int k_
       const int tok = idx / COLS, c = idx % COLS;
       const int jc = blockIdx.x * COLS + c;
       const bool ok = tok < CHUNK && tb + tok < t1 && jc < dv;
-      rv[r] = ok ? rv_to_float(rows[(long long)(tb + tok) * ld + v_col + (long long)h * dv + jc]) : (jc == dv ? 1.0f : 0.f);
+      rv[r] = rows[(long long)(ok ? tb + tok : t0) * ld + v_col + (long long)h * dv + (ok ? jc : 0)];
     }
     const int tok = lane / 2;
-    if (lane < CHUNK * 2 && tb + tok < t1) rg = gates[((long long)(tb + tok) * heads + h) * 3 + lane % 2];
+    const bool ok = lane < CHUNK * 2 && tb + tok < t1;
+    rg = gates[((long long)(ok ? tb + tok : t0) * heads + h) * 3 + lane % 2];
   };
-  auto stage = [&]() {
+  auto stage = [&](int tb) {  // what fetch(tb) brought
 #pragma unroll
     for (int r = 0; r < NK; ++r) {
       const int idx = r * RV_WAVE + lane;
-      if (idx < CHUNK * DKP) (&sk[0][0])[idx] = rk[r], (&sq[0][0])[idx] = rq[r];
+      const int tok = idx / DKP, i = idx % DKP;
+      const bool ok = tok < CHUNK && tb + tok < t1 && i < dk;
+      if (idx < CHUNK * DKP) {
+        (&sk[0][0])[idx] = ok ? rv_to_float(rk[r]) : 0.f;
+        (&sq[0][0])[idx] = ok ? rv_to_float(rq[r]) * q_scale : 0.f;
+      }
     }
 #pragma unroll
     for (int r = 0; r < NV; ++r) {
       const int idx = r * RV_WAVE + lane;
-      if (idx < CHUNK * COLS) (&sv[0][0])[idx] = rv[r];
+      const int tok = idx / COLS, c = idx % COLS;
+      const int jc = blockIdx.x * COLS + c;
+      const bool ok = tok < CHUNK && tb + tok < t1 && jc < dv;
+      if (idx < CHUNK * COLS) (&sv[0][0])[idx] = ok ? rv_to_float(rv[r]) : (jc == dv ? 1.0f : 0.f);
     }
     if (lane < CHUNK * 2) (&sg[0][0])[lane] = rg;
   };
   if (t0 < t1) fetch(t0);
   for (int tb = t0; tb < t1; tb += CHUNK) {
     __syncthreads();  // the chunk before has been read
-    stage();
+    stage(tb);
     __syncthreads();
     if (tb + CHUNK < t1) fetch(tb + CHUNK);
     const int n = min(CHUNK, t1 - tb);
@@ -216,10 +233,7 @@ memory_matrix_kernel(const T* __restrict__ rows, long long ld, int q_col, int k_
         o = fmaf(S[e], qq[e], o);
       }
       o = rg_group_sum<LANES>(o);
-      if (col && sub == 0) {
-        if (is_n) dots[(long long)(tb + t) * heads + h] = o;
-        else out[(long long)(tb + t) * heads * dv + (long long)h * dv + j] = o;
-      }
+      if (col && sub == 0) dst[(long long)(tb + t) * dst_stride] = o;
     }
   }
   if (col) {

@@ -22,7 +22,16 @@ __device__ __forceinline__ float sn_branch(const void* p, int slices, long long 
   if (slices == 0) return rv_to_float(((const T*)p)[at]);
   const float* q = (const float*)p + at;
   float v = 0.f;
-  for (int s = 0; s < slices; ++s) v += q[(size_t)s * stride];
+  int s = 0;
+  for (; s + 4 <= slices; s += 4) {  // four reads on their way at a time; the sums in the slices' order as ever
+    const float a = q[(size_t)s * stride], b = q[(size_t)(s + 1) * stride], c = q[(size_t)(s + 2) * stride],
+                d = q[(size_t)(s + 3) * stride];
+    v += a;
+    v += b;
+    v += c;
+    v += d;
+  }
+  for (; s < slices; ++s) v += q[(size_t)s * stride];
   return v;
 }
 
