@@ -207,7 +207,58 @@ __global__ void __launch_bounds__(SN_THREADS) streams_update_kernel(StreamsParam
     if (P.total) P.total[row0 + i] = all;
     return in_sum;
   };
-  if constexpr (E > 0) {
+  if constexpr (E > 0 && ST > 0) {
+    // a few streams and a row that the registers hold: everything a thread's elements need is asked for first (the
+    // old streams, the branch with all its slices), then worked on, so that the reads of one element do not wait
+    // behind the writes of the one before
+    float olds[E][SMAX], ys[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const int i = e * SN_THREADS + threadIdx.x;
+      ys[e] = 0.f;
+#pragma unroll
+      for (int s = 0; s < SMAX; ++s) olds[e][s] = 0.f;
+      if (i < width) {
+#pragma unroll
+        for (int s = 0; s < SMAX; ++s)
+          olds[e][s] = P.seed ? P.seed[row0 + i] : P.streams[(size_t)s * P.stream_stride + row0 + i];
+        if (P.branch) {
+          float y = sn_branch<T>(P.branch, P.slices, P.slice_stride, row0 + i);
+          if (P.branch2) y = P.wa * y + P.wb * sn_branch<T>(P.branch2, P.slices2, P.slice_stride2, row0 + i);
+          if (P.layer_scale) y *= P.layer_scale[i];
+          ys[e] = y;
+        }
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const int i = e * SN_THREADS + threadIdx.x;
+      u[e] = 0.f;
+      if (i < width) {
+        float fresh[SMAX];
+#pragma unroll
+        for (int t = 0; t < SMAX; ++t) {
+          if (P.branch) {
+            float acc = 0.f;
+#pragma unroll
+            for (int s2 = 0; s2 < SMAX; ++s2) acc = fmaf(s_mix[s2 * S + t], olds[e][s2], acc);
+            fresh[t] = fmaf(s_out[t], ys[e], acc);
+          } else {
+            fresh[t] = olds[e][t];
+          }
+        }
+        float in_sum = 0.f, all = 0.f;
+#pragma unroll
+        for (int s2 = 0; s2 < SMAX; ++s2) {
+          if (P.branch || P.seed) P.streams[(size_t)s2 * P.stream_stride + row0 + i] = fresh[s2];
+          in_sum = fmaf(s_in[s2], fresh[s2], in_sum);
+          all += fresh[s2];
+        }
+        if (P.total) P.total[row0 + i] = all;
+        u[e] = in_sum;
+      }
+    }
+  } else if constexpr (E > 0) {
 #pragma unroll
     for (int e = 0; e < E; ++e) {
       const int i = e * SN_THREADS + threadIdx.x;
