@@ -1,5 +1,5 @@
 """rvllm_amd: a single-GPU inference engine for decoder-only language models (the
-Gemma dense text decoder, the Pinorax and Rufedra designs) on AMD MI355X (gfx950).
+Gemma dense text decoder, the Pinorax, Rufedra and Dafalix designs) on AMD MI355X (gfx950).
 
     import rvllm_amd
     out = rvllm_amd.generate("path/to/model", [[2, 17, 5]], max_tokens=32)
